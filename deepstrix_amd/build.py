@@ -1,0 +1,47 @@
+"""Compiles the HIP sources of this package for gfx950 into deepstrix_amd/lib/*.so.
+
+hipcc cross-compiles without a GPU.  The libraries are built in-tree so that a copy of the
+repository carries them; nothing is compiled at import time.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG, "csrc")
+LIB = os.path.join(PKG, "lib")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+]
+
+TARGETS = {
+    "libdsx_moe.so": ["dsx_api.hip"],
+    "libdsx_synth.so": ["dsx_synth.hip"],
+}
+
+
+def build_all(verbose: bool = False) -> None:
+    os.makedirs(LIB, exist_ok=True)
+    for out, srcs in TARGETS.items():
+        cmd = [HIPCC, *FLAGS, "-o", os.path.join(LIB, out)] + [os.path.join(CSRC, s) for s in srcs]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        # the host pass does not know the gfx feature flag and says so; everything else is shown
+        noise = "is not a recognized feature for this target"
+        text = "\n".join(l for l in res.stdout.splitlines() if noise not in l)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {out}:\n{text}")
+        if text.strip():
+            print(text, file=sys.stderr)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)

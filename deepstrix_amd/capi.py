@@ -1,0 +1,115 @@
+"""ctypes binding of libdsx_moe.so (include/dsx_moe.h).
+
+This is the stand-in for the reference's Rust FFI layer (crates/v4flash-hip/src/sys.rs):
+plain pointers and sizes in, an int status out, mapped to an exception the way the Rust
+wrappers map a status to eyre::Report (crates/v4flash-hip/src/error.rs:10-78).  There is no
+fallback: if the library is missing the import fails.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG, "lib", "libdsx_moe.so")
+
+FMT_Q8_0 = 8
+FMT_MXFP4 = 39
+ROUTER_SQRT_SOFTPLUS, ROUTER_SIGMOID, ROUTER_SOFTMAX = 0, 1, 2
+ERR_INVALID_ARG, ERR_SHAPE, ERR_UNSUPPORTED, ERR_DEVICE = -1, -2, -3, -4
+Q8K_BLOCK_BYTES = 292
+MXFP4_SUPER_BYTES = 136
+
+
+class DsxError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"dsx error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class LayerDesc(C.Structure):
+    _fields_ = [
+        ("hidden", C.c_uint32), ("inter", C.c_uint32), ("n_expert", C.c_uint32),
+        ("n_used", C.c_uint32),
+        ("gate_fmt", C.c_int), ("up_fmt", C.c_int), ("down_fmt", C.c_int),
+        ("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p),
+        ("gate_bpe", C.c_uint64), ("up_bpe", C.c_uint64), ("down_bpe", C.c_uint64),
+        ("clamp", C.c_float),
+        ("router_mode", C.c_uint32), ("n_group", C.c_uint32), ("topk_group", C.c_uint32),
+        ("route_scale", C.c_float), ("route_eps", C.c_float),
+        ("bias", C.c_void_p),
+        ("sh_inter", C.c_uint32),
+        ("sh_gate_fmt", C.c_int), ("sh_up_fmt", C.c_int), ("sh_down_fmt", C.c_int),
+        ("sh_gate", C.c_void_p), ("sh_up", C.c_void_p), ("sh_down", C.c_void_p),
+        ("sh_clamp", C.c_float),
+    ]
+
+
+_vp, _u32, _u64, _f32, _int, _sz = C.c_void_p, C.c_uint32, C.c_uint64, C.c_float, C.c_int, C.c_size_t
+
+# name -> (restype, argtypes); every symbol include/dsx_moe.h declares
+SIGNATURES = {
+    "dsx_abi_version": (_int, []),
+    "dsx_last_error": (C.c_char_p, []),
+    "dsx_init": (_int, []),
+    "dsx_router_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _f32, _u32, _u32, _u32, _u32]),
+    "dsx_q8k_quantize": (_int, [_vp, _vp, _vp, _u32]),
+    "dsx_q8_0_quantize": (_int, [_vp, _vp, _vp, _vp, _u32]),
+    "dsx_q8_0_quantize_rows": (_int, [_vp, _vp, _vp, _u32, _u32]),
+    "dsx_moe_gate_up_batch": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _u64, _u32, _f32, _u32, _u32]),
+    "dsx_moe_down_batched": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _u64, _u32, _u32, _u32, _u32]),
+    "dsx_moe_group_build": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32]),
+    "dsx_moe_gate_up_chunked_rows": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                            _u32, _u64, _u64, _u32, _u32, _f32, _u32, _u32]),
+    "dsx_moe_down_by_expert": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u64,
+                                      _u32, _u32, _u32, _u32, _u32]),
+    "dsx_moe_reduce_partials": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "dsx_dense_ffn_scratch_bytes": (_sz, [_u32, _u32, _u32]),
+    "dsx_dense_ffn": (_int, [_vp, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _f32, _int, _vp]),
+    "dsx_vec_add_inplace": (_int, [_vp, _vp, _vp, _u64]),
+    "dsx_rms_norm": (_int, [_vp, _vp, _vp, _vp, _u32, _f32, _u32]),
+    "dsx_swiglu_clamp_weighted": (_int, [_vp, _vp, _vp, _vp, _vp, _f32, _u32, _u32]),
+    "dsx_mxfp4_repack_hf_to_v2": (_int, [_vp, _vp, _vp, _vp, _u32, _u32]),
+    "dsx_dequant_rows": (_int, [_vp, _int, _vp, _vp, _u32, _u32]),
+    "dsx_moe_layer_create": (_int, [C.POINTER(LayerDesc), C.POINTER(_vp)]),
+    "dsx_moe_layer_destroy": (None, [_vp]),
+    "dsx_moe_layer_workspace_bytes": (_sz, [_vp, _u32]),
+    "dsx_moe_layer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _sz, _vp, _vp, _vp, _vp]),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Loads the library (raises if it was not built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m deepstrix_amd.build` "
+                "(there is no CPU fallback)")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise DsxError(rc, lib().dsx_last_error().decode("utf-8", "replace"))
+
+
+_inited = set()
+
+
+def init() -> None:
+    """Verifies the current device is gfx950 (once per device)."""
+    import torch
+    dev = torch.cuda.current_device()
+    if dev not in _inited:
+        check(lib().dsx_init())
+        _inited.add(dev)

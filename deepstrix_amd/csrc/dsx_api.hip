@@ -1,0 +1,454 @@
+// dsx_api.hip -- the C ABI of libdsx_moe.so (see include/dsx_moe.h): argument validation,
+// grid/block selection and the layer-level sequencing.  Nothing here synchronizes,
+// allocates device memory or reads back, so every entry point can be captured in a graph.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+#include "../../include/dsx_moe.h"
+#include "dsx_expert_kernels.hpp"
+#include "dsx_misc_kernels.hpp"
+#include "dsx_q8_0_kernels.hpp"
+
+using namespace dsx;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int launched(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "%s: %s", what, hipGetErrorString(e));
+    return DSX_OK;
+}
+
+hipStream_t S(dsx_stream_t s) { return (hipStream_t)s; }
+
+bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+// Kernels whose dynamic LDS may exceed the 64 KiB default get their limit raised once.
+template <typename K>
+void allow_lds(K kernel) {
+    (void)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024 - 16 * 1024);
+}
+
+std::once_flag g_attr_once;
+void raise_lds_limits() {
+    std::call_once(g_attr_once, [] {
+        allow_lds(k_mxfp4_gate_up<1, false>);
+        allow_lds(k_mxfp4_gate_up<1, true>);
+        allow_lds(k_mxfp4_gate_up<2, true>);
+        allow_lds(k_mxfp4_gate_up<4, true>);
+        allow_lds(k_mxfp4_gate_up<8, true>);
+        allow_lds(k_mxfp4_down_decode);
+        allow_lds(k_mxfp4_down_by_expert<1>);
+        allow_lds(k_mxfp4_down_by_expert<2>);
+        allow_lds(k_mxfp4_down_by_expert<4>);
+        allow_lds(k_mxfp4_down_by_expert<8>);
+        allow_lds(k_mxfp4_down_by_expert<16>);
+        q8_0_raise_lds_limits();
+    });
+}
+
+constexpr size_t kLdsBudget = 140 * 1024;  // dynamic LDS a workgroup may ask for
+
+int pick_nt(uint32_t chunk) {
+    if (chunk <= 1) return 1;
+    if (chunk <= 2) return 2;
+    if (chunk <= 4) return 4;
+    if (chunk <= 8) return 8;
+    return 16;
+}
+
+template <int NT>
+static void launch_gate_up_be(hipStream_t st, const GateUpParams &p, uint32_t max_wi, size_t lds) {
+    hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true>), dim3(p.n_rows / 16, max_wi),
+                       dim3(kGuWaves * 64), lds, st, p);
+}
+
+template <int NT>
+static void launch_down_be(hipStream_t st, const DownByExpertParams &p, uint32_t max_wi, size_t lds) {
+    hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT>), dim3(p.n_rows / 16, max_wi),
+                       dim3(kDownBeWaves * 64), lds, st, p);
+}
+
+}  // namespace
+
+int dsx::q8_0_unsupported(const char *what) {
+    return fail(DSX_ERR_UNSUPPORTED, "%s: Q8_0 expert kernels are not built", what);
+}
+
+extern "C" {
+
+int dsx_abi_version(void) { return DSX_ABI_VERSION; }
+
+const char *dsx_last_error(void) { return g_err; }
+
+int dsx_init(void) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "dsx_init: hipGetDevice: %s", hipGetErrorString(e));
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess)
+        return fail((int)e, "dsx_init: hipGetDeviceProperties: %s", hipGetErrorString(e));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(DSX_ERR_DEVICE, "dsx_init: device %d is %s; this library is built for gfx950",
+                    dev, prop.gcnArchName);
+    raise_lds_limits();
+    return DSX_OK;
+}
+
+// ---- router -------------------------------------------------------------------------
+int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, const float *logits,
+                    const float *bias, uint32_t n_expert, uint32_t n_used, float scale, float eps,
+                    uint32_t b, uint32_t mode, uint32_t n_group, uint32_t topk_group) {
+    if (b == 0) return DSX_OK;
+    if (!selected || !weights || !logits) return fail(DSX_ERR_INVALID_ARG, "router_topk: null pointer");
+    if (n_expert == 0 || n_expert > DSX_MAX_EXPERTS)
+        return fail(DSX_ERR_INVALID_ARG, "router_topk: n_expert=%u not in 1..%d", n_expert,
+                    DSX_MAX_EXPERTS);
+    if (n_used == 0 || n_used > DSX_MAX_USED || n_used > n_expert)
+        return fail(DSX_ERR_INVALID_ARG, "router_topk: n_used=%u not in 1..%d", n_used, DSX_MAX_USED);
+    if (mode > 2) return fail(DSX_ERR_INVALID_ARG, "router_topk: mode=%u", mode);
+    if (n_group > 1) {
+        if (n_group > 64 || n_expert % n_group != 0 || topk_group == 0)
+            return fail(DSX_ERR_SHAPE, "router_topk: n_group=%u topk_group=%u n_expert=%u", n_group,
+                        topk_group, n_expert);
+    }
+    hipLaunchKernelGGL(k_router_topk, dim3(b), dim3(64), 0, S(stream), selected, weights, logits,
+                       bias, n_expert, n_used, scale, eps, mode, n_group, topk_group);
+    return launched("router_topk");
+}
+
+// ---- quantizers -----------------------------------------------------------------------
+int dsx_q8k_quantize(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t n_blocks) {
+    if (n_blocks == 0) return DSX_OK;
+    if (!out || !x) return fail(DSX_ERR_INVALID_ARG, "q8k_quantize: null pointer");
+    if (!aligned(x, 16) || !aligned(out, 4))
+        return fail(DSX_ERR_SHAPE, "q8k_quantize: x must be 16-byte and out 4-byte aligned");
+    hipLaunchKernelGGL(k_q8k_quantize, dim3((n_blocks + 3) / 4), dim3(256), 0, S(stream), out, x,
+                       n_blocks);
+    return launched("q8k_quantize");
+}
+
+int dsx_q8_0_quantize(dsx_stream_t stream, int8_t *xq, float *xscale, const float *x,
+                      uint32_t blocks) {
+    if (blocks == 0) return DSX_OK;
+    if (!xq || !xscale || !x) return fail(DSX_ERR_INVALID_ARG, "q8_0_quantize: null pointer");
+    if (!aligned(x, 16) || !aligned(xq, 4))
+        return fail(DSX_ERR_SHAPE, "q8_0_quantize: x must be 16-byte and xq 4-byte aligned");
+    hipLaunchKernelGGL(k_q8_0_quantize, dim3((blocks * 8 + 255) / 256), dim3(256), 0, S(stream), xq,
+                       xscale, x, blocks);
+    return launched("q8_0_quantize");
+}
+
+int dsx_q8_0_quantize_rows(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t rows,
+                           uint32_t k) {
+    if (rows == 0) return DSX_OK;
+    if (!out || !x) return fail(DSX_ERR_INVALID_ARG, "q8_0_quantize_rows: null pointer");
+    if (k == 0 || k % 32 != 0) return fail(DSX_ERR_SHAPE, "q8_0_quantize_rows: k=%u must be a multiple of 32", k);
+    if (!aligned(x, 16) || !aligned(out, 4))
+        return fail(DSX_ERR_SHAPE, "q8_0_quantize_rows: x must be 16-byte and out 4-byte aligned");
+    const uint64_t threads = (uint64_t)rows * (k / 32) * 8;
+    hipLaunchKernelGGL(k_q8_0_quantize_rows, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0,
+                       S(stream), out, x, rows, k);
+    return launched("q8_0_quantize_rows");
+}
+
+// ---- decode ---------------------------------------------------------------------------
+static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint8_t *gate,
+                               const uint8_t *up, const uint8_t *xq, const float *ew,
+                               const int32_t *selected, const uint8_t *sh_gate,
+                               const uint8_t *sh_up, float sh_clamp, uint64_t gbpe, uint64_t ubpe,
+                               uint32_t n_used, float clamp, uint32_t n_rows, uint32_t n_blocks) {
+    if (n_used == 0 && !sh_gate) return DSX_OK;
+    if (!mid || !gate || !up || !xq || !ew || !selected)
+        return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: null pointer");
+    if (n_used > DSX_MAX_USED) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: n_used=%u", n_used);
+    if (dtype == DSX_FMT_Q8_0)
+        return q8_0_gate_up_decode(st, mid, gate, up, xq, ew, selected, sh_gate, sh_up, sh_clamp,
+                                   gbpe, ubpe, n_used, clamp, n_rows, n_blocks);
+    if (dtype != DSX_FMT_MXFP4)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_batch: no kernel for dtype %d", dtype);
+    if (n_rows == 0 || n_rows % 16 != 0)
+        return fail(DSX_ERR_SHAPE, "moe_gate_up_batch: n_rows=%u must be a multiple of 16", n_rows);
+    if (n_blocks == 0) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: n_blocks=0");
+    if (gbpe % 8 || ubpe % 8 || !aligned(gate, 8) || !aligned(up, 8) || !aligned(xq, 4))
+        return fail(DSX_ERR_SHAPE, "moe_gate_up_batch: weights must be 8-byte aligned, xq 4-byte");
+    const size_t lds = (size_t)n_blocks * 512 + (size_t)n_blocks * 4;
+    if (lds > kLdsBudget)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_batch: n_blocks=%u exceeds LDS staging", n_blocks);
+    raise_lds_limits();
+    GateUpParams p{};
+    p.mid = mid; p.gate = gate; p.up = up; p.xq = xq; p.ew = ew; p.selected = selected;
+    p.sh_gate = sh_gate; p.sh_up = sh_up; p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used;
+    p.chunk = 1; p.clamp = clamp; p.sh_clamp = sh_clamp; p.n_rows = n_rows; p.n_blocks = n_blocks;
+    p.xq_row_bytes = n_blocks * kQ8kBytes;
+    const uint32_t n_slots = n_used + (sh_gate ? 1u : 0u);
+    hipLaunchKernelGGL((k_mxfp4_gate_up<1, false>), dim3(n_rows / 16, n_slots), dim3(kGuWaves * 64),
+                       lds, st, p);
+    return launched("moe_gate_up_batch");
+}
+
+int dsx_moe_gate_up_batch(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
+                          const uint8_t *up, const uint8_t *xq, const float *ew,
+                          const int32_t *selected, uint64_t gbpe, uint64_t ubpe, uint32_t n_used,
+                          float clamp, uint32_t n_rows, uint32_t n_blocks) {
+    return gate_up_decode_impl(S(stream), dtype, mid, gate, up, xq, ew, selected, nullptr, nullptr,
+                               0.0f, gbpe, ubpe, n_used, clamp, n_rows, n_blocks);
+}
+
+static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t *down,
+                            const uint8_t *xq, const int32_t *selected, const uint8_t *sh_down,
+                            uint64_t dbpe, uint32_t xq_slot_stride, uint32_t n_used,
+                            uint32_t n_rows, uint32_t n_blocks_in) {
+    if (!out || !down || !xq || !selected)
+        return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: null pointer");
+    if (n_used > DSX_MAX_USED) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_used=%u", n_used);
+    if (dtype == DSX_FMT_Q8_0)
+        return q8_0_down_decode(st, out, down, xq, selected, sh_down, dbpe, xq_slot_stride, n_used,
+                                n_rows, n_blocks_in);
+    if (dtype != DSX_FMT_MXFP4)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_down_batched: no kernel for dtype %d", dtype);
+    if (n_rows == 0 || n_rows % 16 != 0)
+        return fail(DSX_ERR_SHAPE, "moe_down_batched: n_rows=%u must be a multiple of 16", n_rows);
+    if (n_blocks_in == 0) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_blocks_in=0");
+    if (xq_slot_stride < n_blocks_in * kQ8kBytes || xq_slot_stride % 4)
+        return fail(DSX_ERR_SHAPE, "moe_down_batched: xq_slot_stride=%u", xq_slot_stride);
+    if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, 4))
+        return fail(DSX_ERR_SHAPE, "moe_down_batched: weights must be 8-byte aligned, xq 4-byte");
+    const uint32_t n_slots = n_used + (sh_down ? 1u : 0u);
+    const size_t units = (size_t)n_slots * n_blocks_in;
+    const size_t lds = units * 512 + units * 4;
+    if (lds > kLdsBudget)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_down_batched: %zu (slot, block) tiles exceed LDS", units);
+    raise_lds_limits();
+    DownDecodeParams p{};
+    p.out = out; p.down = down; p.xq = xq; p.selected = selected; p.sh_down = sh_down;
+    p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.n_slots = n_slots;
+    p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
+    hipLaunchKernelGGL(k_mxfp4_down_decode, dim3(n_rows / 16), dim3(kDownWaves * 64), lds, st, p);
+    return launched("moe_down_batched");
+}
+
+int dsx_moe_down_batched(dsx_stream_t stream, int dtype, float *out, const uint8_t *down,
+                         const uint8_t *xq, const int32_t *selected, uint64_t dbpe,
+                         uint32_t xq_slot_stride, uint32_t n_used, uint32_t n_rows,
+                         uint32_t n_blocks_in) {
+    if (n_used == 0) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_used=0");
+    return down_decode_impl(S(stream), dtype, out, down, xq, selected, nullptr, dbpe,
+                            xq_slot_stride, n_used, n_rows, n_blocks_in);
+}
+
+// ---- by-expert ------------------------------------------------------------------------
+int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,
+                        int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
+                        const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
+                        uint32_t chunk) {
+    if (!group_count || !group_offset || !expert_members || !work_items || !n_work_items || !selected)
+        return fail(DSX_ERR_INVALID_ARG, "moe_group_build: null pointer");
+    if (n_expert == 0 || n_expert > DSX_MAX_EXPERTS)
+        return fail(DSX_ERR_INVALID_ARG, "moe_group_build: n_expert=%u", n_expert);
+    if (b >= 65536 || n_used == 0 || n_used >= 65536)
+        return fail(DSX_ERR_INVALID_ARG, "moe_group_build: b=%u n_used=%u must be below 65536", b, n_used);
+    if (chunk == 0 || chunk > 16) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..16", chunk);
+    hipLaunchKernelGGL(k_group_build, dim3(1), dim3(kGbThreads), 0, S(stream), group_count,
+                       group_offset, expert_members, work_items, n_work_items, selected, b, n_used,
+                       n_expert, chunk);
+    return launched("moe_group_build");
+}
+
+int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
+                                 const uint8_t *up, const uint8_t *xq, const float *ew,
+                                 const int32_t *group_count, const int32_t *group_offset,
+                                 const int32_t *expert_members, const int32_t *work_items,
+                                 const int32_t *n_work_items, uint32_t max_work_items,
+                                 uint64_t gbpe, uint64_t ubpe, uint32_t n_used, uint32_t chunk,
+                                 float clamp, uint32_t n_rows, uint32_t n_blocks) {
+    if (max_work_items == 0) return DSX_OK;
+    if (!mid || !gate || !up || !xq || !ew || !group_count || !group_offset || !expert_members ||
+        !work_items || !n_work_items)
+        return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: null pointer");
+    if (max_work_items > 65535)
+        return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: max_work_items=%u", max_work_items);
+    if (chunk == 0 || chunk > 16) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: chunk=%u", chunk);
+    if (dtype == DSX_FMT_Q8_0)
+        return q8_0_gate_up_by_expert(S(stream), mid, gate, up, xq, ew, group_count, group_offset,
+                                      expert_members, work_items, n_work_items, max_work_items,
+                                      gbpe, ubpe, n_used, chunk, clamp, n_rows, n_blocks);
+    if (dtype != DSX_FMT_MXFP4)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows: no kernel for dtype %d", dtype);
+    if (n_rows == 0 || n_rows % 16 != 0)
+        return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: n_rows=%u must be a multiple of 16", n_rows);
+    if (n_blocks == 0) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: n_blocks=0");
+    if (gbpe % 8 || ubpe % 8 || !aligned(gate, 8) || !aligned(up, 8) || !aligned(xq, 4))
+        return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: weights must be 8-byte aligned, xq 4-byte");
+    const int nt = pick_nt(chunk);
+    const size_t lds = (size_t)n_blocks * 512 * nt + (size_t)n_blocks * nt * 4;
+    if (lds > kLdsBudget || nt > 8)
+        return fail(DSX_ERR_UNSUPPORTED,
+                    "moe_gate_up_chunked_rows: chunk=%u x n_blocks=%u needs %zu B of LDS", chunk,
+                    n_blocks, lds);
+    raise_lds_limits();
+    GateUpParams p{};
+    p.mid = mid; p.gate = gate; p.up = up; p.xq = xq; p.ew = ew;
+    p.group_count = group_count; p.group_offset = group_offset; p.members = expert_members;
+    p.work_items = work_items; p.n_work_items = n_work_items;
+    p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used; p.chunk = chunk; p.clamp = clamp;
+    p.n_rows = n_rows; p.n_blocks = n_blocks; p.xq_row_bytes = n_blocks * kQ8kBytes;
+    hipStream_t st = S(stream);
+    switch (nt) {
+        case 1: launch_gate_up_be<1>(st, p, max_work_items, lds); break;
+        case 2: launch_gate_up_be<2>(st, p, max_work_items, lds); break;
+        case 4: launch_gate_up_be<4>(st, p, max_work_items, lds); break;
+        default: launch_gate_up_be<8>(st, p, max_work_items, lds); break;
+    }
+    return launched("moe_gate_up_chunked_rows");
+}
+
+int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, const uint8_t *down,
+                           const uint8_t *xq, const int32_t *group_count,
+                           const int32_t *group_offset, const int32_t *expert_members,
+                           const int32_t *work_items, const int32_t *n_work_items,
+                           uint32_t max_work_items, uint64_t dbpe, uint32_t xq_slot_stride,
+                           uint32_t n_used, uint32_t chunk, uint32_t n_rows, uint32_t n_blocks_in) {
+    if (max_work_items == 0) return DSX_OK;
+    if (!partials || !down || !xq || !group_count || !group_offset || !expert_members ||
+        !work_items || !n_work_items)
+        return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: null pointer");
+    if (max_work_items > 65535)
+        return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: max_work_items=%u", max_work_items);
+    if (chunk == 0 || chunk > 16) return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: chunk=%u", chunk);
+    if (dtype == DSX_FMT_Q8_0)
+        return q8_0_down_by_expert(S(stream), partials, down, xq, group_count, group_offset,
+                                   expert_members, work_items, n_work_items, max_work_items, dbpe,
+                                   xq_slot_stride, n_used, chunk, n_rows, n_blocks_in);
+    if (dtype != DSX_FMT_MXFP4)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert: no kernel for dtype %d", dtype);
+    if (n_rows == 0 || n_rows % 16 != 0)
+        return fail(DSX_ERR_SHAPE, "moe_down_by_expert: n_rows=%u must be a multiple of 16", n_rows);
+    if (n_blocks_in == 0) return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: n_blocks_in=0");
+    if (xq_slot_stride < n_blocks_in * kQ8kBytes || xq_slot_stride % 4)
+        return fail(DSX_ERR_SHAPE, "moe_down_by_expert: xq_slot_stride=%u", xq_slot_stride);
+    if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, 4))
+        return fail(DSX_ERR_SHAPE, "moe_down_by_expert: weights must be 8-byte aligned, xq 4-byte");
+    const int nt = pick_nt(chunk);
+    const size_t lds = (size_t)n_blocks_in * 512 * nt + (size_t)n_blocks_in * nt * 4;
+    if (lds > kLdsBudget)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert: chunk=%u x n_blocks_in=%u needs %zu B of LDS",
+                    chunk, n_blocks_in, lds);
+    raise_lds_limits();
+    DownByExpertParams p{};
+    p.partials = partials; p.down = down; p.xq = xq;
+    p.group_count = group_count; p.group_offset = group_offset; p.members = expert_members;
+    p.work_items = work_items; p.n_work_items = n_work_items;
+    p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk;
+    p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
+    hipStream_t st = S(stream);
+    switch (nt) {
+        case 1: launch_down_be<1>(st, p, max_work_items, lds); break;
+        case 2: launch_down_be<2>(st, p, max_work_items, lds); break;
+        case 4: launch_down_be<4>(st, p, max_work_items, lds); break;
+        case 8: launch_down_be<8>(st, p, max_work_items, lds); break;
+        default: launch_down_be<16>(st, p, max_work_items, lds); break;
+    }
+    return launched("moe_down_by_expert");
+}
+
+static int reduce_impl(hipStream_t st, float *out, const float *partials, const int32_t *selected,
+                       const float *add, uint32_t n_used, uint32_t n_rows, uint32_t b) {
+    if (b == 0) return DSX_OK;
+    if (!out || !partials) return fail(DSX_ERR_INVALID_ARG, "moe_reduce_partials: null pointer");
+    if (n_rows == 0 || n_rows % 4 != 0 || !aligned(out, 16) || !aligned(partials, 16) ||
+        (add && !aligned(add, 16)))
+        return fail(DSX_ERR_SHAPE, "moe_reduce_partials: n_rows=%u must be a multiple of 4, buffers 16-byte aligned", n_rows);
+    const uint64_t n4 = (uint64_t)b * (n_rows / 4);
+    hipLaunchKernelGGL(k_reduce_partials, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, st, out,
+                       partials, selected, add, n_used, n_rows, b);
+    return launched("moe_reduce_partials");
+}
+
+int dsx_moe_reduce_partials(dsx_stream_t stream, float *out, const float *partials,
+                            const int32_t *selected, uint32_t n_used, uint32_t n_rows, uint32_t b) {
+    return reduce_impl(S(stream), out, partials, selected, nullptr, n_used, n_rows, b);
+}
+
+// ---- element-wise -----------------------------------------------------------------------
+int dsx_vec_add_inplace(dsx_stream_t stream, float *out, const float *rhs, uint64_t n) {
+    if (n == 0) return DSX_OK;
+    if (!out || !rhs) return fail(DSX_ERR_INVALID_ARG, "vec_add_inplace: null pointer");
+    hipLaunchKernelGGL(k_vec_add_inplace, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, S(stream),
+                       out, rhs, n);
+    return launched("vec_add_inplace");
+}
+
+int dsx_rms_norm(dsx_stream_t stream, float *out, const float *x, const float *weight, uint32_t n,
+                 float eps, uint32_t rows) {
+    if (rows == 0) return DSX_OK;
+    if (!out || !x || !weight || n == 0) return fail(DSX_ERR_INVALID_ARG, "rms_norm: null pointer or n=0");
+    hipLaunchKernelGGL(k_rms_norm, dim3(rows), dim3(256), 0, S(stream), out, x, weight, n, eps);
+    return launched("rms_norm");
+}
+
+int dsx_swiglu_clamp_weighted(dsx_stream_t stream, float *mid, const float *gate, const float *up,
+                              const float *expert_w, float clamp, uint32_t ff, uint32_t n_experts) {
+    if (ff == 0 || n_experts == 0) return DSX_OK;
+    if (!mid || !gate || !up || !expert_w)
+        return fail(DSX_ERR_INVALID_ARG, "swiglu_clamp_weighted: null pointer");
+    hipLaunchKernelGGL(k_swiglu_clamp_weighted, dim3((ff + 255) / 256, n_experts), dim3(256), 0,
+                       S(stream), mid, gate, up, expert_w, clamp, ff);
+    return launched("swiglu_clamp_weighted");
+}
+
+// ---- weight pipeline ----------------------------------------------------------------------
+int dsx_mxfp4_repack_hf_to_v2(dsx_stream_t stream, uint8_t *dst, const uint8_t *packed,
+                              const uint8_t *scale, uint32_t out, uint32_t nb) {
+    if (out == 0 || nb == 0) return DSX_OK;
+    if (!dst || !packed || !scale) return fail(DSX_ERR_INVALID_ARG, "mxfp4_repack: null pointer");
+    if (nb % 8 != 0) return fail(DSX_ERR_SHAPE, "mxfp4_repack: nb=%u must be a multiple of 8", nb);
+    if (!aligned(dst, 8) || !aligned(packed, 8))
+        return fail(DSX_ERR_SHAPE, "mxfp4_repack: dst and packed must be 8-byte aligned");
+    const uint64_t n = (uint64_t)out * nb;
+    hipLaunchKernelGGL(k_mxfp4_repack, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, S(stream),
+                       dst, packed, scale, out, nb);
+    return launched("mxfp4_repack");
+}
+
+int dsx_dequant_rows(dsx_stream_t stream, int dtype, float *y, const uint8_t *rows, uint32_t n_rows,
+                     uint32_t cols) {
+    if (n_rows == 0 || cols == 0) return DSX_OK;
+    if (!y || !rows) return fail(DSX_ERR_INVALID_ARG, "dequant_rows: null pointer");
+    if (dtype == DSX_FMT_MXFP4) {
+        if (cols % 256) return fail(DSX_ERR_SHAPE, "dequant_rows: cols=%u must be a multiple of 256", cols);
+        const uint64_t nb = (uint64_t)n_rows * (cols / 32);
+        hipLaunchKernelGGL(k_mxfp4_dequant, dim3((uint32_t)((nb + 255) / 256)), dim3(256), 0,
+                           S(stream), y, rows, nb);
+    } else if (dtype == DSX_FMT_Q8_0) {
+        if (cols % 32) return fail(DSX_ERR_SHAPE, "dequant_rows: cols=%u must be a multiple of 32", cols);
+        const uint64_t nb = (uint64_t)n_rows * (cols / 32);
+        hipLaunchKernelGGL(k_q8_0_dequant, dim3((uint32_t)((nb + 255) / 256)), dim3(256), 0,
+                           S(stream), y, rows, n_rows, cols / 32);
+    } else {
+        return fail(DSX_ERR_UNSUPPORTED, "dequant_rows: dtype %d", dtype);
+    }
+    return launched("dequant_rows");
+}
+
+}  // extern "C"
+
+#include "dsx_layer.inc"

@@ -1,0 +1,172 @@
+// dsx_device.hpp -- device-side building blocks shared by the gfx950 MoE kernels.
+//
+// The expert products run on the CDNA4 block-scaled matrix instruction
+// V_MFMA_SCALE_F32_16X16X128_F8F6F4.  One instruction multiplies a 16-row x 128-k tile
+// of FP4 (E2M1) weights, each 32-k block carrying its own E8M0 scale, with a 128-k x
+// 16-column tile of FP8 (E4M3) activations.  That is exactly the shape of the engine's
+// MXFP4 data: a lane's A operand is one 16-byte nibble block of a 136-byte super-block,
+// loaded with a single 128-bit global load and never decoded on the vector ALU.
+//
+// The reference multiplies MXFP4 weights with int8 (Q8_K) activations
+// (crates/v4flash-kernels/src/mxfp4_tables.rs:49-74).  int8 is not an MFMA operand type
+// next to FP4, so each activation q is split exactly as q + 128 = 16*uh + ul with
+// uh, ul in [0, 15]:   q = 16*(uh - 8) + ul.   Both (uh - 8) and ul are small integers
+// that E4M3 holds exactly; the "high" plane is multiplied by 2^4 through the B-side
+// block scale.  Every product is exact and the block sums are exact in f32, so the
+// result is the reference's integer dot product, accumulated in f32.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dsx {
+
+constexpr int kSuperBytes = 136;   // MXFP4 super-block: 8 x 16 B nibbles + 8 scale bytes
+constexpr int kQ8kBytes = 292;     // f32 d | i8 qs[256] | i16 bsums[16]
+constexpr int kTileBytes1 = 512;   // staged activation bytes per (super-block, token): 2 planes x 256
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct __attribute__((packed, aligned(8))) U4A8 {
+    uint32_t x, y, z, w;
+};
+struct __attribute__((packed, aligned(4))) U2A4 {
+    uint32_t x, y;
+};
+
+// E4M3 (OCP) byte of a small non-negative integer m in [0, 15].
+__device__ __forceinline__ uint32_t e4m3_of_uint(uint32_t m) {
+    // 0,1,2,3,4,5,6,7 -> 0x00,0x38,0x40,0x44,0x48,0x4A,0x4C,0x4E ; 8..15 -> 0x50 | (m & 7)
+    const uint32_t lo = 0x44403800u, hi = 0x4E4C4A48u;
+    const uint32_t t = (m & 4u) ? hi : lo;
+    const uint32_t small = (t >> ((m & 3u) * 8u)) & 0xFFu;
+    return (m & 8u) ? (0x50u | (m & 7u)) : small;
+}
+
+// int8 q -> (high plane byte, low plane byte):  q = 16 * hi + lo, hi in [-8, 7], lo in [0, 15].
+__device__ __forceinline__ void split_q(int q, uint32_t &hi_byte, uint32_t &lo_byte) {
+    const uint32_t u = (uint32_t)(q + 128) & 0xFFu;
+    const uint32_t ul = u & 15u, uh = u >> 4;
+    lo_byte = e4m3_of_uint(ul);
+    const bool neg = uh < 8u;
+    const uint32_t mag = neg ? (8u - uh) : (uh - 8u);
+    hi_byte = e4m3_of_uint(mag) | (neg ? 0x80u : 0u);
+}
+
+// ---------------------------------------------------------------------------------------
+// Staged activation tile in LDS, for one super-block (256 k) and NT token columns.
+//
+// The MFMA's B operand gives lane l column (l % 16) and the 32-k block (l / 16) of a 128-k
+// half, 32 bytes in k order.  The weights' nibble byte j holds element j (low nibble) and
+// element 16 + j (high nibble) of the block, so MFMA position p of a block is element
+// p/2 (p even) or 16 + p/2 (p odd); the activation bytes are stored in that order.
+//
+//   tile[half h][plane][chunk c][kb][column][16 B]     half = block/4, kb = block%4,
+//   plane 0 = high (x16), plane 1 = low, chunk c = positions 16c .. 16c+15.
+// A lane reads its operand as two 16-byte chunks; consecutive lanes read consecutive
+// 16-byte words (NT == 16) or broadcast (NT < 16).
+// ---------------------------------------------------------------------------------------
+template <int NT>
+__device__ __forceinline__ uint32_t tile_off(uint32_t h, uint32_t plane, uint32_t c, uint32_t kb,
+                                             uint32_t col) {
+    return (((((h * 2u + plane) * 2u + c) * 4u + kb) * NT) + col) * 16u;
+}
+
+// One wave converts one Q8_K block (292 B in global memory) into the tile of column `col`.
+// lane -> (block b32 = lane / 8, dword d = lane % 8); dword d holds positions 4d..4d+3 =
+// elements (2d, 16+2d, 2d+1, 17+2d) of the block.
+template <int NT>
+__device__ __forceinline__ void stage_q8k_block(uint8_t *tile, float *yd_slot,
+                                                const uint8_t *__restrict__ blk, uint32_t col,
+                                                uint32_t lane) {
+    const uint32_t b32 = lane >> 3, d = lane & 7u;
+    const int8_t *q8 = (const int8_t *)(blk + 4) + b32 * 32u;
+    const uint16_t lo2 = *(const uint16_t *)(q8 + 2u * d);
+    const uint16_t hi2 = *(const uint16_t *)(q8 + 16u + 2u * d);
+    const int q0 = (int8_t)(lo2 & 0xFF), q2 = (int8_t)(lo2 >> 8);
+    const int q1 = (int8_t)(hi2 & 0xFF), q3 = (int8_t)(hi2 >> 8);
+    uint32_t h0, l0, h1, l1, h2, l2, h3, l3;
+    split_q(q0, h0, l0);
+    split_q(q1, h1, l1);
+    split_q(q2, h2, l2);
+    split_q(q3, h3, l3);
+    const uint32_t hw = h0 | (h1 << 8) | (h2 << 16) | (h3 << 24);
+    const uint32_t lw = l0 | (l1 << 8) | (l2 << 16) | (l3 << 24);
+    const uint32_t h = b32 >> 2, kb = b32 & 3u, c = d >> 2, o = (d & 3u) * 4u;
+    *(uint32_t *)(tile + tile_off<NT>(h, 0, c, kb, col) + o) = hw;
+    *(uint32_t *)(tile + tile_off<NT>(h, 1, c, kb, col) + o) = lw;
+    if (lane == 0) *yd_slot = *(const float *)blk;
+}
+
+// Weights of one super-block for the lane's row: its two nibble blocks (halves 0 and 1,
+// block kb of each) and the 8 scale bytes.
+struct WSuper {
+    U4A8 a0, a1;
+    U2A4 s;
+};
+
+__device__ __forceinline__ WSuper load_wsuper(const uint8_t *__restrict__ row_super, uint32_t kb) {
+    WSuper w;
+    w.a0 = *(const U4A8 *)(row_super + kb * 16u);
+    w.a1 = *(const U4A8 *)(row_super + 64u + kb * 16u);
+    w.s = *(const U2A4 *)(row_super + 128u);
+    return w;
+}
+
+__device__ __forceinline__ v8i b_operand(const uint8_t *tile, uint32_t off0, uint32_t off1) {
+    const uint4 lo = *(const uint4 *)(tile + off0);
+    const uint4 hi = *(const uint4 *)(tile + off1);
+    v8i b = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    return b;
+}
+
+// The lane's four B operands of one super-block: {high, low} plane x {half 0, half 1}.
+struct BSuper {
+    v8i h0, l0, h1, l1;
+};
+
+template <int NT>
+__device__ __forceinline__ BSuper load_bsuper(const uint8_t *tile, uint32_t kb, uint32_t col) {
+    BSuper b;
+    b.h0 = b_operand(tile, tile_off<NT>(0, 0, 0, kb, col), tile_off<NT>(0, 0, 1, kb, col));
+    b.l0 = b_operand(tile, tile_off<NT>(0, 1, 0, kb, col), tile_off<NT>(0, 1, 1, kb, col));
+    b.h1 = b_operand(tile, tile_off<NT>(1, 0, 0, kb, col), tile_off<NT>(1, 0, 1, kb, col));
+    b.l1 = b_operand(tile, tile_off<NT>(1, 1, 0, kb, col), tile_off<NT>(1, 1, 1, kb, col));
+    return b;
+}
+
+// acc[i] += yd * sum_k W[row][k] * q[k]   over one super-block, for the lane's 4 rows
+// (4 * (lane / 16) + i) and its column (lane % 16).  Scale bytes: the weights' E8M0 as
+// stored (2^(e-127) on E2M1 == 2^(e-128) on the doubled kvalues), 131 (2^4) for the
+// activation high plane, 127 (2^0) for the low plane.
+__device__ __forceinline__ void mfma_super(v4f &acc, const WSuper &w, const BSuper &b, float yd,
+                                           uint32_t kb) {
+    const v8i a0 = {(int)w.a0.x, (int)w.a0.y, (int)w.a0.z, (int)w.a0.w, 0, 0, 0, 0};
+    const v8i a1 = {(int)w.a1.x, (int)w.a1.y, (int)w.a1.z, (int)w.a1.w, 0, 0, 0, 0};
+    const int s0 = (int)((w.s.x >> (kb * 8u)) & 0xFFu);
+    const int s1 = (int)((w.s.y >> (kb * 8u)) & 0xFFu);
+    v4f c = {0.f, 0.f, 0.f, 0.f};
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a0, b.h0, c, 4, 0, 0, s0, 0, 131);
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a0, b.l0, c, 4, 0, 0, s0, 0, 127);
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a1, b.h1, c, 4, 0, 0, s1, 0, 131);
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a1, b.l1, c, 4, 0, 0, s1, 0, 127);
+    acc.x = fmaf(yd, c.x, acc.x);
+    acc.y = fmaf(yd, c.y, acc.y);
+    acc.z = fmaf(yd, c.z, acc.z);
+    acc.w = fmaf(yd, c.w, acc.w);
+}
+
+// crates/v4flash-kernels/kernels/swiglu_clamp_weighted.hip:27-36
+__device__ __forceinline__ float swiglu_clamp(float g, float u, float clamp, float ew) {
+    if (clamp > 1.0e-6f) {
+        if (g > clamp) g = clamp;
+        if (u > clamp) u = clamp;
+        if (u < -clamp) u = -clamp;
+    }
+    const float sig = 1.0f / (1.0f + expf(-g));
+    return g * sig * u * ew;
+}
+
+}  // namespace dsx

@@ -1,0 +1,556 @@
+// dsx_misc_kernels.hpp -- router, activation quantizers, token->expert inversion,
+// reductions and the small element-wise kernels of the MoE path (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dsx_device.hpp"
+
+namespace dsx {
+
+// 64-lane butterfly reductions.  Every lane ends with the full result.
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint64_t other = __shfl_xor(v, o, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Order-preserving map f32 -> u32 (larger float => larger integer).
+__device__ __forceinline__ uint32_t f32_key(float f) {
+    const uint32_t b = __float_as_uint(f);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// ---------------------------------------------------------------------------------------
+// Router.  One wave per token; lane l owns experts l, l+64, ...  (n_expert <= 512).
+//   p      = sqrt(softplus(logit)) | sigmoid(logit) | softmax(logits)
+//   score  = p + bias, then group-limited masking
+//   k passes of arg-max over score (ties -> lowest index), winner masked to -inf
+//   w_j    = p[sel_j] / max(sum_j p[sel_j], eps) * scale
+// crates/v4flash-kernels/kernels/router_topk.hip:32-36,70-131,
+// crates/v4flash-kernels/kernels/laguna_ops.hip:395-451.
+// ---------------------------------------------------------------------------------------
+constexpr int kRouterPerLane = 8;  // 512 / 64
+
+__device__ __forceinline__ float softplus_stable(float x) {
+    if (x > 20.0f) return x;
+    if (x < -20.0f) return expf(x);
+    return log1pf(expf(x));
+}
+
+__global__ __launch_bounds__(64) void k_router_topk(int32_t *__restrict__ selected,
+                                                    float *__restrict__ weights,
+                                                    const float *__restrict__ logits,
+                                                    const float *__restrict__ bias,
+                                                    uint32_t n_expert, uint32_t n_used, float scale,
+                                                    float eps, uint32_t mode, uint32_t n_group,
+                                                    uint32_t topk_group) {
+    __shared__ float s_score[512];
+    __shared__ float s_gscore[64];
+    __shared__ int s_keep[64];
+
+    const uint32_t t = blockIdx.x, lane = threadIdx.x;
+    const float *lg = logits + (uint64_t)t * n_expert;
+
+    float p[kRouterPerLane], s[kRouterPerLane];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; j++) {
+        const uint32_t e = lane + 64u * j;
+        p[j] = (e < n_expert) ? lg[e] : -INFINITY;
+        mx = fmaxf(mx, p[j]);
+    }
+    if (mode == 2u) {  // softmax
+        mx = wave_max_f32(mx);
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) {
+            const uint32_t e = lane + 64u * j;
+            p[j] = (e < n_expert) ? expf(p[j] - mx) : 0.0f;
+            sum += p[j];
+        }
+        sum = wave_sum_f32(sum);
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) p[j] = p[j] / sum;
+    } else {
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) {
+            const uint32_t e = lane + 64u * j;
+            if (e < n_expert)
+                p[j] = (mode == 0u) ? sqrtf(softplus_stable(p[j])) : 1.0f / (1.0f + expf(-p[j]));
+            else
+                p[j] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; j++) {
+        const uint32_t e = lane + 64u * j;
+        s[j] = (e < n_expert) ? ((bias != nullptr) ? p[j] + bias[e] : p[j]) : -INFINITY;
+    }
+
+    if (n_group > 1u && topk_group < n_group) {
+        // group score = sum of the two largest biased scores of the group
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) {
+            const uint32_t e = lane + 64u * j;
+            if (e < n_expert) s_score[e] = s[j];
+        }
+        __syncthreads();
+        const uint32_t gs = n_expert / n_group;
+        if (lane < n_group) {
+            float a = -INFINITY, b = -INFINITY;
+            for (uint32_t i = 0; i < gs; i++) {
+                const float v = s_score[lane * gs + i];
+                if (v > a) {
+                    b = a;
+                    a = v;
+                } else if (v > b) {
+                    b = v;
+                }
+            }
+            s_gscore[lane] = (gs >= 2u) ? a + b : a;
+        }
+        __syncthreads();
+        if (lane < n_group) {
+            // rank among groups: better = larger score, ties -> lower index
+            const float mine = s_gscore[lane];
+            uint32_t rank = 0;
+            for (uint32_t g = 0; g < n_group; g++) {
+                const float o = s_gscore[g];
+                rank += (o > mine || (o == mine && g < lane)) ? 1u : 0u;
+            }
+            s_keep[lane] = rank < topk_group ? 1 : 0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) {
+            const uint32_t e = lane + 64u * j;
+            if (e < n_expert && !s_keep[e / gs]) s[j] = -INFINITY;
+        }
+    }
+
+    float sum = 0.0f;
+    float my_p = 0.0f;  // lane k keeps the k-th pick's unbiased p
+    int my_sel = -1;
+    for (uint32_t k = 0; k < n_used; k++) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) {
+            const uint32_t e = lane + 64u * j;
+            if (e < n_expert) {
+                const uint64_t key = ((uint64_t)f32_key(s[j]) << 32) | (uint64_t)(0xFFFFFFFFu - e);
+                best = key > best ? key : best;
+            }
+        }
+        best = wave_max_u64(best);
+        // nothing left above -inf: an empty pick (p = 0), as a scan with `>` would leave it
+        const bool none = (uint32_t)(best >> 32) <= f32_key(-INFINITY);
+        const uint32_t e_win = 0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFu);
+        const uint32_t owner = e_win & 63u, jj = e_win >> 6;
+        float pw = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++) {
+            if ((uint32_t)j == jj) {
+                pw = p[j];
+                if (lane == owner && !none) s[j] = -INFINITY;
+            }
+        }
+        pw = none ? 0.0f : __shfl(pw, (int)owner, 64);
+        sum += pw;  // every lane adds the same values in pick order
+        if (lane == k) {
+            my_p = pw;
+            my_sel = none ? -1 : (int)e_win;
+        }
+    }
+    if (sum < eps) sum = eps;
+    if (lane < n_used) {
+        selected[(uint64_t)t * n_used + lane] = my_sel;
+        weights[(uint64_t)t * n_used + lane] = my_p / sum * scale;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Q8_K quantizer: one wave per 256-element block, 4 consecutive elements per lane.
+// crates/v4flash-kernels/kernels/q8_k_quantize.hip:23-90
+// ---------------------------------------------------------------------------------------
+struct Q8kQuant {
+    float d;       // 1 / iscale (0 for an all-zero block)
+    int q[4];      // the lane's four quantized values
+};
+
+__device__ __forceinline__ Q8kQuant q8k_quantize_lane(float4 v, uint32_t lane) {
+    // key = (|x| bits, 255 - index): the largest |x| wins, the first one on ties
+    const float xs[4] = {v.x, v.y, v.z, v.w};
+    uint64_t best = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t idx = lane * 4u + i;
+        const uint64_t key = ((uint64_t)(__float_as_uint(xs[i]) & 0x7FFFFFFFu) << 32) | (255u - idx);
+        best = key > best ? key : best;
+    }
+    best = wave_max_u64(best);
+    const uint32_t amax_bits = (uint32_t)(best >> 32);
+    const uint32_t idx = 255u - (uint32_t)(best & 0xFFu);
+    float cand = xs[0];
+    if ((idx & 3u) == 1u) cand = xs[1];
+    if ((idx & 3u) == 2u) cand = xs[2];
+    if ((idx & 3u) == 3u) cand = xs[3];
+    const float mxv = __shfl(cand, (int)(idx >> 2), 64);
+    Q8kQuant r;
+    if (amax_bits == 0u) {
+        r.d = 0.0f;
+        r.q[0] = r.q[1] = r.q[2] = r.q[3] = 0;
+        return r;
+    }
+    const float iscale = -127.0f / mxv;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int q = (int)rintf(iscale * xs[i]);
+        q = q > 127 ? 127 : q;
+        q = q < -128 ? -128 : q;
+        r.q[i] = q;
+    }
+    r.d = 1.0f / iscale;
+    return r;
+}
+
+__global__ __launch_bounds__(256) void k_q8k_quantize(uint8_t *__restrict__ out,
+                                                      const float *__restrict__ x,
+                                                      uint32_t n_blocks) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t b = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (b >= n_blocks) return;
+    const float4 v = *(const float4 *)(x + (uint64_t)b * 256u + lane * 4u);
+    const Q8kQuant r = q8k_quantize_lane(v, lane);
+    uint8_t *blk = out + (uint64_t)b * kQ8kBytes;
+    const uint32_t packed = (uint32_t)(r.q[0] & 0xFF) | ((uint32_t)(r.q[1] & 0xFF) << 8) |
+                            ((uint32_t)(r.q[2] & 0xFF) << 16) | ((uint32_t)(r.q[3] & 0xFF) << 24);
+    *(uint32_t *)(blk + 4u + lane * 4u) = packed;
+    int s = r.q[0] + r.q[1] + r.q[2] + r.q[3];
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    if ((lane & 3u) == 0u) *(int16_t *)(blk + 260u + (lane >> 2) * 2u) = (int16_t)s;
+    if (lane == 0) *(float *)blk = r.d;
+}
+
+// Q8_0 activation quantizer: 8 lanes per 32-element block, 4 elements per lane.
+// crates/v4flash-kernels/kernels/q8_0_matvec.hip:150-177
+__global__ __launch_bounds__(256) void k_q8_0_quantize(int8_t *__restrict__ xq,
+                                                       float *__restrict__ xscale,
+                                                       const float *__restrict__ x,
+                                                       uint32_t blocks) {
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t b = gid >> 3, sub = gid & 7u;
+    const bool live = b < blocks;
+    float4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) v = *(const float4 *)(x + (uint64_t)b * 32u + sub * 4u);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    if (!live) return;
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float xs[4] = {v.x, v.y, v.z, v.w};
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int q = (int)rintf(xs[i] * id);
+        q = q > 127 ? 127 : q;
+        q = q < -128 ? -128 : q;
+        packed |= (uint32_t)(q & 0xFF) << (8 * i);
+    }
+    *(uint32_t *)(xq + (uint64_t)b * 32u + sub * 4u) = packed;
+    if (sub == 0) xscale[b] = d;
+}
+
+// ---------------------------------------------------------------------------------------
+// Token -> expert inversion: histogram, exclusive prefix sum, stable scatter, work items.
+// One workgroup of 1024 threads (b * n_used and n_expert are small next to the expert
+// products).  Members of an expert are in ascending (token, slot) order and work items in
+// ascending (expert, start) order, so the result is the same on every run.
+// Replaces crates/v4flash-kernels/kernels/moe_group_builder.hip:32-51 and
+// moe_work_items_builder.hip:26-44 (atomic order, dense [n_expert x max] table).
+// ---------------------------------------------------------------------------------------
+constexpr int kGbThreads = 1024;
+#define DSX_MAX_EXPERTS_K 512
+
+__global__ __launch_bounds__(kGbThreads) void k_group_build(
+    int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
+    int32_t *__restrict__ members, int32_t *__restrict__ work_items,
+    int32_t *__restrict__ n_work_items, const int32_t *__restrict__ selected, uint32_t b,
+    uint32_t n_used, uint32_t n_expert, uint32_t chunk) {
+    __shared__ int s_count[DSX_MAX_EXPERTS_K];
+    __shared__ int s_off[DSX_MAX_EXPERTS_K + 1];
+    __shared__ int s_wi_off[DSX_MAX_EXPERTS_K + 1];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t total = b * n_used;
+    for (uint32_t e = tid; e < n_expert; e += kGbThreads) s_count[e] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < total; i += kGbThreads) {
+        const int e = selected[i];
+        if (e >= 0 && (uint32_t)e < n_expert) atomicAdd(&s_count[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int acc = 0, wacc = 0;
+        for (uint32_t e = 0; e < n_expert; e++) {
+            s_off[e] = acc;
+            s_wi_off[e] = wacc;
+            acc += s_count[e];
+            wacc += (s_count[e] + (int)chunk - 1) / (int)chunk;
+        }
+        s_off[n_expert] = acc;
+        s_wi_off[n_expert] = wacc;
+        *n_work_items = wacc;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < n_expert; e += kGbThreads) {
+        group_count[e] = s_count[e];
+        group_offset[e] = s_off[e];
+        const int nwi = s_wi_off[e + 1] - s_wi_off[e];
+        for (int c = 0; c < nwi; c++)
+            work_items[s_wi_off[e] + c] = (int)((e << 16) | ((uint32_t)c * chunk));
+    }
+    if (tid == 0) group_offset[n_expert] = s_off[n_expert];
+    // stable scatter: a wave owns experts wave, wave + 16, ...; it walks the picks 64 at
+    // a time and places the matching ones with a ballot prefix count.
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    for (uint32_t e = wave; e < n_expert; e += kGbThreads / 64) {
+        if (s_count[e] == 0) continue;
+        uint32_t pos = (uint32_t)s_off[e];
+        for (uint32_t i0 = 0; i0 < total; i0 += 64u) {
+            const uint32_t i = i0 + lane;
+            const bool hit = (i < total) && (selected[i] == (int)e);
+            const uint64_t mask = __ballot(hit);
+            if (hit) {
+                const uint32_t before = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+                const uint32_t t = i / n_used, slot = i - t * n_used;
+                members[pos + before] = (int)((t << 16) | slot);
+            }
+            pos += (uint32_t)__popcll(mask);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// out[t, row] = sum over slots of partials[(t * n_used + s) * n_rows + row], in slot order.
+// crates/v4flash-kernels/kernels/q2_k_accumulate_matvec_par.hip:714-730
+// `selected` (nullable): slots with a negative pick are skipped.
+// `add` (nullable): added last (the shared expert, crates/v4flash-kernels/kernels/vec_add.hip:6-13).
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_reduce_partials(float *__restrict__ out,
+                                                         const float *__restrict__ partials,
+                                                         const int32_t *__restrict__ selected,
+                                                         const float *__restrict__ add,
+                                                         uint32_t n_used, uint32_t n_rows,
+                                                         uint32_t b) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;  // float4 index
+    const uint64_t per_row = n_rows / 4u;
+    if (i >= (uint64_t)b * per_row) return;
+    const uint64_t t = i / per_row, c = i - t * per_row;
+    float4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t s = 0; s < n_used; s++) {
+        if (selected != nullptr && selected[t * n_used + s] < 0) continue;
+        const float4 v = *(const float4 *)(partials + ((t * n_used + s) * n_rows) + c * 4u);
+        acc.x += v.x;
+        acc.y += v.y;
+        acc.z += v.z;
+        acc.w += v.w;
+    }
+    if (add != nullptr) {
+        const float4 v = *(const float4 *)(add + t * n_rows + c * 4u);
+        acc.x += v.x;
+        acc.y += v.y;
+        acc.z += v.z;
+        acc.w += v.w;
+    }
+    *(float4 *)(out + t * n_rows + c * 4u) = acc;
+}
+
+// crates/v4flash-kernels/kernels/vec_add.hip:6-13
+__global__ __launch_bounds__(256) void k_vec_add_inplace(float *__restrict__ out,
+                                                         const float *__restrict__ rhs,
+                                                         uint64_t n) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n) out[i] += rhs[i];
+}
+
+// crates/v4flash-kernels/kernels/swiglu_clamp_weighted.hip:16-37
+__global__ __launch_bounds__(256) void k_swiglu_clamp_weighted(float *__restrict__ mid,
+                                                               const float *__restrict__ gate,
+                                                               const float *__restrict__ up,
+                                                               const float *__restrict__ expert_w,
+                                                               float clamp, uint32_t ff) {
+    const uint32_t r = blockIdx.x * 256u + threadIdx.x;
+    if (r >= ff) return;
+    const uint32_t e = blockIdx.y;
+    const uint64_t idx = (uint64_t)e * ff + r;
+    mid[idx] = swiglu_clamp(gate[idx], up[idx], clamp, expert_w[e]);
+}
+
+// RMS norm, one workgroup per row: 256 strided f64 partial sums, f32 tree, then scale.
+// crates/v4flash-kernels/kernels/rms_norm.hip:12-50
+__global__ __launch_bounds__(256) void k_rms_norm(float *__restrict__ out,
+                                                  const float *__restrict__ x,
+                                                  const float *__restrict__ weight, uint32_t n,
+                                                  float eps) {
+    __shared__ float sdata[256];
+    const uint32_t tid = threadIdx.x;
+    const float *xr = x + (uint64_t)blockIdx.x * n;
+    float *orow = out + (uint64_t)blockIdx.x * n;
+    double partial = 0.0;
+    for (uint32_t i = tid; i < n; i += 256u) {
+        const float v = xr[i];
+        partial += (double)v * (double)v;
+    }
+    sdata[tid] = (float)partial;
+    __syncthreads();
+    for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+        if (tid < stride) sdata[tid] += sdata[tid + stride];
+        __syncthreads();
+    }
+    const float mean_sq = sdata[0] / (float)n;
+    const float scale = 1.0f / sqrtf(mean_sq + eps);
+    for (uint32_t i = tid; i < n; i += 256u) orow[i] = xr[i] * scale * weight[i];
+}
+
+// HF packed nibbles + E8M0 scales -> v2 super-block rows, one thread per 32-element block.
+// crates/v4flash-kernels/kernels/mxfp4_repack.hip:35-65 (same bytes as
+// crates/v4flash-core/src/hf_v41.rs:1208-1232).
+__global__ __launch_bounds__(256) void k_mxfp4_repack(uint8_t *__restrict__ dst,
+                                                      const uint8_t *__restrict__ packed,
+                                                      const uint8_t *__restrict__ scale,
+                                                      uint32_t out, uint32_t nb) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= (uint64_t)out * nb) return;
+    const uint64_t r = i / nb, j = i - r * nb;
+    const uint8_t *pb = packed + (r * nb + j) * 16u;
+    uint8_t *sup = dst + r * nb * 17u + (j >> 3) * 136u;
+    const uint32_t k = (uint32_t)(j & 7u);
+    sup[128u + k] = scale[r * nb + j];
+    const uint2 lo = *(const uint2 *)pb, hi = *(const uint2 *)(pb + 8);
+    const uint8_t *lob = (const uint8_t *)&lo, *hib = (const uint8_t *)&hi;
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t l8 = lob[2 * q + h], h8 = hib[2 * q + h];
+            const uint32_t b0 = (l8 & 0x0Fu) | ((h8 << 4) & 0xF0u);
+            const uint32_t b1 = (l8 >> 4) | (h8 & 0xF0u);
+            v |= (b0 | (b1 << 8)) << (16 * h);
+        }
+        w[q] = v;
+    }
+    uint2 *d2 = (uint2 *)(sup + k * 16u);
+    d2[0] = make_uint2(w[0], w[1]);
+    d2[1] = make_uint2(w[2], w[3]);
+}
+
+// Dequantize engine rows to f32 (checking aid).
+__device__ __forceinline__ float e8m0_half(uint32_t e) {
+    return __uint_as_float((e < 2u) ? (0x00200000u << e) : ((e - 1u) << 23));
+}
+__global__ __launch_bounds__(256) void k_mxfp4_dequant(float *__restrict__ y,
+                                                       const uint8_t *__restrict__ rows,
+                                                       uint64_t n_blocks32) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= n_blocks32) return;
+    const int8_t kv[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+    const uint8_t *sup = rows + (i >> 3) * 136u;
+    const uint32_t k = (uint32_t)(i & 7u);
+    const float d = e8m0_half(sup[128u + k]);
+    for (int j = 0; j < 16; j++) {
+        const uint8_t q = sup[k * 16u + j];
+        y[i * 32u + j] = (float)kv[q & 15u] * d;
+        y[i * 32u + 16u + j] = (float)kv[q >> 4] * d;
+    }
+}
+__global__ __launch_bounds__(256) void k_q8_0_dequant(float *__restrict__ y,
+                                                      const uint8_t *__restrict__ rows,
+                                                      uint32_t n_rows, uint32_t blocks) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= (uint64_t)n_rows * blocks) return;
+    const uint64_t r = i / blocks, b = i - r * blocks;
+    const uint8_t *wr = rows + r * blocks * 34u;
+    const float d = __half2float(*(const __half *)(wr + b * 2u));
+    const int8_t *q = (const int8_t *)(wr + (uint64_t)blocks * 2u + b * 32u);
+    for (int j = 0; j < 32; j++) y[i * 32u + j] = d * (float)q[j];
+}
+
+// Identity grouping for a dense expert: every token is a member of expert 0 with weight 1.
+__global__ __launch_bounds__(256) void k_dense_groups(int32_t *__restrict__ group_count,
+                                                      int32_t *__restrict__ group_offset,
+                                                      int32_t *__restrict__ members,
+                                                      int32_t *__restrict__ work_items,
+                                                      int32_t *__restrict__ n_work_items,
+                                                      float *__restrict__ ones, uint32_t b,
+                                                      uint32_t chunk) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < b) {
+        members[i] = (int)(i << 16);
+        ones[i] = 1.0f;
+    }
+    const uint32_t nwi = (b + chunk - 1) / chunk;
+    if (i < nwi) work_items[i] = (int)(i * chunk);
+    if (i == 0) {
+        group_count[0] = (int)b;
+        group_offset[0] = 0;
+        group_offset[1] = (int)b;
+        *n_work_items = (int)nwi;
+    }
+}
+
+// Q8_0 activation rows: [k int8][k/32 f32 scales], one row per token
+// (same arithmetic as k_q8_0_quantize; the scales follow the quants so that one pointer
+// names a token's activation, like a Q8_K row does).
+__global__ __launch_bounds__(256) void k_q8_0_quantize_rows(uint8_t *__restrict__ out,
+                                                            const float *__restrict__ x,
+                                                            uint32_t rows, uint32_t k) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint32_t bpr = k / 32u;
+    const uint64_t blk = gid >> 3;
+    const uint32_t sub = (uint32_t)(gid & 7u);
+    const bool live = blk < (uint64_t)rows * bpr;
+    const uint64_t r = live ? blk / bpr : 0, b = live ? blk - r * bpr : 0;
+    float4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) v = *(const float4 *)(x + r * k + b * 32u + sub * 4u);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    if (!live) return;
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float xs[4] = {v.x, v.y, v.z, v.w};
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int q = (int)rintf(xs[i] * id);
+        q = q > 127 ? 127 : q;
+        q = q < -128 ? -128 : q;
+        packed |= (uint32_t)(q & 0xFF) << (8 * i);
+    }
+    uint8_t *row = out + r * (uint64_t)(k + k / 8u);
+    *(uint32_t *)(row + b * 32u + sub * 4u) = packed;
+    if (sub == 0) *(float *)(row + k + b * 4u) = d;
+}
+
+}  // namespace dsx

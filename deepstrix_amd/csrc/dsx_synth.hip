@@ -1,0 +1,225 @@
+// dsx_synth.hip -- counter-based synthetic tensors for benchmarks and tests (libdsx_synth.so).
+//
+// Not part of the MoE operator ABI.  Every value is a pure function of
+// (seed, tensor id, element index), computed with integer arithmetic only, so the host
+// loops and the device kernels below produce the same bytes and any slice of a tensor
+// (one expert, one row) can be generated on its own.
+//
+//   h(c)      = splitmix64(base + c),  base = splitmix64(seed ^ (tensor_id * 0x9E3779B97F4A7C15))
+//   normal(i) = (sum of the twelve 16-bit fields of h(3i), h(3i+1), h(3i+2) - 393210) / 65536
+//               (Irwin-Hall of order 12: mean 0, variance 1, support +-6)
+// Weights: normal * sigma, quantized to MXFP4 (E2M1 x E8M0 per 32, scale =
+// 2^ceil(log2(amax/6)), nearest code with ties to the even code) in the engine's
+// super-block layout, or to Q8_0 rows ([blocks x f16 d][blocks x 32 i8], d = amax/127,
+// q = round-half-away(x / d)).
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+#define HD __host__ __device__ __forceinline__
+
+namespace {
+
+HD uint64_t splitmix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+HD uint64_t stream_base(uint64_t seed, uint64_t tensor_id) {
+    return splitmix64(seed ^ (tensor_id * 0x9E3779B97F4A7C15ull));
+}
+
+HD uint32_t sum16(uint64_t h) {
+    return (uint32_t)(h & 0xFFFF) + (uint32_t)((h >> 16) & 0xFFFF) + (uint32_t)((h >> 32) & 0xFFFF) +
+           (uint32_t)(h >> 48);
+}
+
+HD float normal_at(uint64_t base, uint64_t i) {
+    const uint32_t s = sum16(splitmix64(base + 3 * i)) + sum16(splitmix64(base + 3 * i + 1)) +
+                       sum16(splitmix64(base + 3 * i + 2));
+    return (float)((int32_t)s - 393210) * (1.0f / 65536.0f);
+}
+
+HD int e2m1_index(float ax) {
+    const float grid[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+    int best = 0;
+    float best_diff = fabsf(ax - grid[0]);
+    for (int i = 1; i < 8; i++) {
+        const float diff = fabsf(ax - grid[i]);
+        if (diff < best_diff || (diff == best_diff && (i & 1) == 0 && (best & 1) != 0)) {
+            best = i;
+            best_diff = diff;
+        }
+    }
+    return best;
+}
+
+// One 32-element block of row-major element index i0 .. i0+31 -> 16 nibble bytes + scale byte.
+HD void mxfp4_block(uint64_t base, uint64_t i0, float sigma, uint8_t *nib16, uint8_t *scale_byte) {
+    float x[32];
+    float amax = 0.0f;
+    for (int j = 0; j < 32; j++) {
+        x[j] = normal_at(base, i0 + j) * sigma;
+        const float a = fabsf(x[j]);
+        if (a > amax) amax = a;
+    }
+    if (amax < 7.052966104933725e-38f) amax = 7.052966104933725e-38f;
+    const float t = amax / 6.0f;
+    int e;
+    const float m = frexpf(t, &e);
+    const int cexp = (m == 0.5f) ? e - 1 : e;
+    const float scale = ldexpf(1.0f, cexp);
+    *scale_byte = (uint8_t)(cexp + 127);
+    uint8_t code[32];
+    for (int j = 0; j < 32; j++) {
+        float q = x[j] / scale;
+        if (q > 6.0f) q = 6.0f;
+        if (q < -6.0f) q = -6.0f;
+        code[j] = (uint8_t)(e2m1_index(fabsf(q)) | ((x[j] < 0.0f) ? 8 : 0));
+    }
+    for (int j = 0; j < 16; j++) nib16[j] = (uint8_t)(code[j] | (code[j + 16] << 4));
+}
+
+HD uint16_t f32_to_f16_bits(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    const uint32_t mant = x & 0x007fffffu;
+    const int exp = (int)((x >> 23) & 0xffu);
+    if (exp == 0xff) return (uint16_t)(sign | 0x7c00u | (mant ? 0x0200u : 0u));
+    const int e = exp - 127 + 15;
+    if (e >= 0x1f) return (uint16_t)(sign | 0x7c00u);
+    if (e <= 0) {
+        if (e < -10) return sign;
+        const uint32_t m = mant | 0x00800000u;
+        const uint32_t shift = (uint32_t)(14 - e);
+        const uint16_t half_mant = (uint16_t)(m >> shift);
+        const uint32_t round_bit = 1u << (shift - 1);
+        uint16_t result = (uint16_t)(sign | half_mant);
+        if ((m & round_bit) && ((m & (round_bit - 1)) || (half_mant & 1))) result++;
+        return result;
+    }
+    const uint16_t half_mant = (uint16_t)(mant >> 13);
+    uint16_t result = (uint16_t)(sign | ((uint16_t)e << 10) | half_mant);
+    if ((mant & 0x1000u) && ((mant & 0x0fffu) || (half_mant & 1))) result++;
+    return result;
+}
+
+// One Q8_0 block: f16 scale bits + 32 int8.
+HD void q8_0_block(uint64_t base, uint64_t i0, float sigma, uint16_t *d_bits, int8_t *q32) {
+    float x[32];
+    float amax = 0.0f;
+    for (int j = 0; j < 32; j++) {
+        x[j] = normal_at(base, i0 + j) * sigma;
+        const float a = fabsf(x[j]);
+        if (a > amax) amax = a;
+    }
+    const float d = amax / 127.0f;
+    const float id = (d == 0.0f) ? 0.0f : 1.0f / d;
+    *d_bits = f32_to_f16_bits(d);
+    for (int j = 0; j < 32; j++) q32[j] = (int8_t)roundf(x[j] * id);
+}
+
+// Block index b (row-major over [n_rows, cols/32]) of a tensor whose first row has global
+// element index elem0.
+HD void mxfp4_store(uint8_t *dst, uint64_t base, uint64_t elem0, uint64_t b, uint32_t cols,
+                    float sigma) {
+    const uint64_t bpr = cols / 32u;
+    const uint64_t r = b / bpr, j = b - r * bpr;
+    uint8_t *sup = dst + r * bpr * 17u + (j >> 3) * 136u;
+    const uint32_t k = (uint32_t)(j & 7u);
+    uint8_t nib[16], sc;
+    mxfp4_block(base, elem0 + r * cols + j * 32u, sigma, nib, &sc);
+    for (int i = 0; i < 16; i++) sup[k * 16u + i] = nib[i];
+    sup[128u + k] = sc;
+}
+
+HD void q8_0_store(uint8_t *dst, uint64_t base, uint64_t elem0, uint64_t b, uint32_t cols,
+                   float sigma) {
+    const uint64_t bpr = cols / 32u;
+    const uint64_t r = b / bpr, j = b - r * bpr;
+    uint8_t *row = dst + r * bpr * 34u;
+    uint16_t d;
+    int8_t q[32];
+    q8_0_block(base, elem0 + r * cols + j * 32u, sigma, &d, q);
+    row[j * 2u] = (uint8_t)(d & 0xff);
+    row[j * 2u + 1] = (uint8_t)(d >> 8);
+    for (int i = 0; i < 32; i++) row[bpr * 2u + j * 32u + i] = (uint8_t)q[i];
+}
+
+__global__ void k_normal(float *out, uint64_t base, uint64_t offset, uint64_t n, float sigma,
+                         float mean) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = normal_at(base, offset + i) * sigma + mean;
+}
+__global__ void k_mxfp4(uint8_t *dst, uint64_t base, uint64_t elem0, uint64_t n_blocks,
+                        uint32_t cols, float sigma) {
+    const uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < n_blocks) mxfp4_store(dst, base, elem0, b, cols, sigma);
+}
+__global__ void k_q8_0(uint8_t *dst, uint64_t base, uint64_t elem0, uint64_t n_blocks,
+                       uint32_t cols, float sigma) {
+    const uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < n_blocks) q8_0_store(dst, base, elem0, b, cols, sigma);
+}
+
+}  // namespace
+
+extern "C" {
+
+// out[i] = normal(offset + i) * sigma + mean   (the multiply-add is two rounded f32 ops)
+void dsx_synth_normal_host(float *out, uint64_t seed, uint64_t tensor_id, uint64_t offset,
+                           uint64_t n, float sigma, float mean) {
+    const uint64_t base = stream_base(seed, tensor_id);
+    for (uint64_t i = 0; i < n; i++) {
+        const float v = normal_at(base, offset + i) * sigma;
+        out[i] = v + mean;
+    }
+}
+
+// n_rows rows of `cols` elements starting at global element index elem0, as MXFP4 rows.
+void dsx_synth_mxfp4_host(uint8_t *dst, uint64_t seed, uint64_t tensor_id, uint64_t elem0,
+                          uint64_t n_rows, uint32_t cols, float sigma) {
+    const uint64_t base = stream_base(seed, tensor_id);
+    const uint64_t nb = n_rows * (cols / 32u);
+    for (uint64_t b = 0; b < nb; b++) mxfp4_store(dst, base, elem0, b, cols, sigma);
+}
+
+void dsx_synth_q8_0_host(uint8_t *dst, uint64_t seed, uint64_t tensor_id, uint64_t elem0,
+                         uint64_t n_rows, uint32_t cols, float sigma) {
+    const uint64_t base = stream_base(seed, tensor_id);
+    const uint64_t nb = n_rows * (cols / 32u);
+    for (uint64_t b = 0; b < nb; b++) q8_0_store(dst, base, elem0, b, cols, sigma);
+}
+
+int dsx_synth_normal_dev(void *stream, float *out, uint64_t seed, uint64_t tensor_id,
+                         uint64_t offset, uint64_t n, float sigma, float mean) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_normal, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, out, stream_base(seed, tensor_id), offset, n, sigma, mean);
+    return (int)hipGetLastError();
+}
+
+int dsx_synth_mxfp4_dev(void *stream, uint8_t *dst, uint64_t seed, uint64_t tensor_id,
+                        uint64_t elem0, uint64_t n_rows, uint32_t cols, float sigma) {
+    const uint64_t nb = n_rows * (cols / 32u);
+    if (nb == 0) return 0;
+    hipLaunchKernelGGL(k_mxfp4, dim3((uint32_t)((nb + 127) / 128)), dim3(128), 0,
+                       (hipStream_t)stream, dst, stream_base(seed, tensor_id), elem0, nb, cols, sigma);
+    return (int)hipGetLastError();
+}
+
+int dsx_synth_q8_0_dev(void *stream, uint8_t *dst, uint64_t seed, uint64_t tensor_id,
+                       uint64_t elem0, uint64_t n_rows, uint32_t cols, float sigma) {
+    const uint64_t nb = n_rows * (cols / 32u);
+    if (nb == 0) return 0;
+    hipLaunchKernelGGL(k_q8_0, dim3((uint32_t)((nb + 127) / 128)), dim3(128), 0,
+                       (hipStream_t)stream, dst, stream_base(seed, tensor_id), elem0, nb, cols, sigma);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,0 +1,110 @@
+"""The whole MoE layer behind one object, modelled on the reference's `MoeExecutor`
+(crates/v4flash-kernels/src/het/remote_experts.rs:7432-7443): it records device pointers and
+dimensions, owns the scratch, and `run` produces f32 [T, hidden].  The sequencing itself
+lives in the library (dsx_moe_layer_forward); this class only holds the buffers.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import capi
+from .capi import FMT_MXFP4, LayerDesc, check, lib
+from .dispatch import matrix_bytes
+
+
+@dataclass
+class LayerWeights:
+    """Device tensors (uint8) in engine layout; `RoutedExpertWeights` in the reference
+    (crates/v4flash-kernels/src/model_weights.rs:41-54)."""
+    hidden: int
+    inter: int
+    n_expert: int
+    n_used: int
+    gate: torch.Tensor
+    up: torch.Tensor
+    down: torch.Tensor
+    gate_fmt: int = FMT_MXFP4
+    up_fmt: int = FMT_MXFP4
+    down_fmt: int = FMT_MXFP4
+    clamp: float = 0.0
+    router_mode: int = capi.ROUTER_SIGMOID
+    n_group: int = 1
+    topk_group: int = 1
+    route_scale: float = 1.0
+    route_eps: float = 1e-20
+    bias: Optional[torch.Tensor] = None
+    sh_inter: int = 0
+    sh_gate: Optional[torch.Tensor] = None
+    sh_up: Optional[torch.Tensor] = None
+    sh_down: Optional[torch.Tensor] = None
+    sh_gate_fmt: int = FMT_MXFP4
+    sh_up_fmt: int = FMT_MXFP4
+    sh_down_fmt: int = FMT_MXFP4
+    sh_clamp: float = 0.0
+
+
+class MoeLayer:
+    def __init__(self, w: LayerWeights, max_tokens: int):
+        capi.init()
+        self.w = w
+        self.max_tokens = max_tokens
+        d = LayerDesc()
+        d.hidden, d.inter, d.n_expert, d.n_used = w.hidden, w.inter, w.n_expert, w.n_used
+        d.gate_fmt, d.up_fmt, d.down_fmt = w.gate_fmt, w.up_fmt, w.down_fmt
+        d.gate, d.up, d.down = w.gate.data_ptr(), w.up.data_ptr(), w.down.data_ptr()
+        d.gate_bpe = matrix_bytes(w.gate_fmt, w.inter, w.hidden)
+        d.up_bpe = matrix_bytes(w.up_fmt, w.inter, w.hidden)
+        d.down_bpe = matrix_bytes(w.down_fmt, w.hidden, w.inter)
+        for name, t, bpe in (("gate", w.gate, d.gate_bpe), ("up", w.up, d.up_bpe),
+                             ("down", w.down, d.down_bpe)):
+            if t.numel() * t.element_size() != bpe * w.n_expert:
+                raise ValueError(f"{name}: {t.numel() * t.element_size()} bytes, expected "
+                                 f"{bpe * w.n_expert}")
+        d.clamp = w.clamp
+        d.router_mode, d.n_group, d.topk_group = w.router_mode, w.n_group, w.topk_group
+        d.route_scale, d.route_eps = w.route_scale, w.route_eps
+        d.bias = w.bias.data_ptr() if w.bias is not None else None
+        d.sh_inter = w.sh_inter
+        if w.sh_inter:
+            d.sh_gate_fmt, d.sh_up_fmt, d.sh_down_fmt = w.sh_gate_fmt, w.sh_up_fmt, w.sh_down_fmt
+            d.sh_gate, d.sh_up, d.sh_down = (w.sh_gate.data_ptr(), w.sh_up.data_ptr(),
+                                             w.sh_down.data_ptr())
+            d.sh_clamp = w.sh_clamp
+        self._desc = d
+        h = C.c_void_p()
+        check(lib().dsx_moe_layer_create(C.byref(d), C.byref(h)))
+        self._h = h
+        self.workspace_bytes = int(lib().dsx_moe_layer_workspace_bytes(h, max_tokens))
+        self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=w.gate.device)
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            lib().dsx_moe_layer_destroy(h)
+            self._h = None
+
+    def run(self, x: torch.Tensor, logits: Optional[torch.Tensor] = None, out=None,
+            selected_in=None, weights_in=None, want_routing=False):
+        """x f32 [T, hidden], logits f32 [T, n_expert] -> out f32 [T, hidden]."""
+        T = x.shape[0]
+        if T > self.max_tokens:
+            raise ValueError(f"{T} tokens > max_tokens={self.max_tokens}")
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        if out is None:
+            out = torch.empty((T, self.w.hidden), dtype=torch.float32, device=x.device)
+        sel_out = w_out = None
+        if want_routing:
+            sel_out = torch.empty((T, self.w.n_used), dtype=torch.int32, device=x.device)
+            w_out = torch.empty((T, self.w.n_used), dtype=torch.float32, device=x.device)
+        p = lambda t: None if t is None else t.data_ptr()
+        check(lib().dsx_moe_layer_forward(
+            self._h, torch.cuda.current_stream().cuda_stream, p(out), p(x), p(logits), T,
+            p(self.workspace), self.workspace_bytes, p(sel_out), p(w_out), p(selected_in),
+            p(weights_in)))
+        if want_routing:
+            return out, sel_out, w_out
+        return out

@@ -1,0 +1,221 @@
+/*
+ * dsx_moe.h -- C ABI of libdsx_moe.so: the deepstrix MoE feed-forward path on gfx950.
+ *
+ * What a host engine binds instead of launching the reference's per-arch code
+ * objects.  Every entry point mirrors one launch wrapper / dispatch function of
+ * the reference (cited per function, paths relative to the reference tree) and
+ * keeps its argument order and meaning; the library owns grid/block selection.
+ *
+ * Conventions
+ *   - all pointers are DEVICE pointers owned by the caller unless stated;
+ *   - `stream` is a hipStream_t passed as void*; nothing synchronizes, allocates
+ *     or reads back, so every call may sit inside a HIP graph capture
+ *     (crates/v4flash-kernels/src/het/dispatch.rs:11-13,622-626);
+ *   - return value: 0 = success, > 0 = the hipError_t of the failed launch,
+ *     < 0 = argument validation error (DSX_ERR_*), raised BEFORE anything is
+ *     launched (crates/v4flash-kernels/src/mxfp4.rs:416-424);
+ *     dsx_last_error() returns the thread's last message;
+ *   - an empty problem (0 tokens / 0 work items) is success
+ *     (crates/v4flash-kernels/src/mxfp4.rs:422-424).
+ *
+ * Weight layouts are the engine's, unchanged:
+ *   MXFP4  rows of 136-byte super-blocks: [8 x 16 B nibbles][8 B E8M0 scales],
+ *          256 elements each; experts contiguous, stride = bytes-per-expert
+ *          (crates/v4flash-kernels/src/mxfp4_tables.rs:10-36)
+ *   Q8_0   rows of [blocks x f16 d][blocks x 32 i8]
+ *          (crates/v4flash-kernels/src/weights.rs:225-240)
+ * Activations: Q8_K blocks, 292 B per 256 elements
+ *          (crates/v4flash-kernels/kernels/q8_k_quantize.hip:9-21).
+ */
+#ifndef DSX_MOE_H
+#define DSX_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DSX_ABI_VERSION 1
+
+/* ggml type ids, as carried by the reference's GgufType
+ * (crates/v4flash-core/src/gguf.rs:569-592). */
+#define DSX_FMT_Q8_0 8
+#define DSX_FMT_MXFP4 39
+
+#define DSX_ROUTER_SQRT_SOFTPLUS 0
+#define DSX_ROUTER_SIGMOID 1
+#define DSX_ROUTER_SOFTMAX 2
+
+#define DSX_OK 0
+#define DSX_ERR_INVALID_ARG (-1) /* null pointer, zero/oversized dimension */
+#define DSX_ERR_SHAPE (-2)       /* divisibility / alignment contract broken */
+#define DSX_ERR_UNSUPPORTED (-3) /* format or size this build has no kernel for */
+#define DSX_ERR_DEVICE (-4)      /* current device is not gfx950 */
+
+#define DSX_Q8K_BLOCK_BYTES 292
+#define DSX_MXFP4_SUPER_BYTES 136
+#define DSX_MAX_EXPERTS 512 /* crates/v4flash-kernels/build.rs:93-97 (ROUTER_MAX_EXPERTS) */
+#define DSX_MAX_USED 16     /* crates/v4flash-kernels/kernels/laguna_ops.hip:20 */
+
+typedef void *dsx_stream_t;
+
+int dsx_abi_version(void);
+const char *dsx_last_error(void);
+/* Checks that the current device is gfx950; call once per device before use. */
+int dsx_init(void);
+
+/* ---- router ---------------------------------------------------------------
+ * RouterTopk::launch_batched_ex (crates/v4flash-kernels/src/router_topk.rs:245-364;
+ * kernels router_topk_par.hip:66-238) and laguna_router_topk_batched
+ * (kernels/laguna_ops.hip:395-451).  selected[b,n_used] i32, weights[b,n_used] f32,
+ * logits[b,n_expert] f32, bias[n_expert] f32 or NULL.  mode = DSX_ROUTER_*.
+ * n_group <= 1 disables group-limited routing; otherwise the n_expert/n_group
+ * wide groups are ranked by the sum of their two largest biased scores and only
+ * the best topk_group groups stay eligible. */
+int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, const float *logits,
+                    const float *bias, uint32_t n_expert, uint32_t n_used, float scale, float eps,
+                    uint32_t b, uint32_t mode, uint32_t n_group, uint32_t topk_group);
+
+/* ---- activation quantizers ------------------------------------------------
+ * Q8KQuantize::launch (crates/v4flash-kernels/src/q8_k.rs:33-104). */
+int dsx_q8k_quantize(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t n_blocks);
+/* Q8_0 input quantizer (crates/v4flash-kernels/kernels/q8_0_matvec.hip:150-177). */
+int dsx_q8_0_quantize(dsx_stream_t stream, int8_t *xq, float *xscale, const float *x,
+                      uint32_t blocks);
+/* Same quantizer, one activation row per token as the expert entry points take it for
+ * a Q8_0 matrix: out[rows] rows of (k + k/8) bytes = [k int8][k/32 f32 scales]. */
+int dsx_q8_0_quantize_rows(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t rows,
+                           uint32_t k);
+
+/* ---- decode (one token) ---------------------------------------------------
+ * dispatch::moe_gate_up_batch (crates/v4flash-kernels/src/het/dispatch.rs:26-66):
+ * mid[slot,row] = swiglu(gate_e[row].xq, up_e[row].xq; clamp) * ew[slot],
+ * e = selected[slot]; mid is [n_used, n_rows] f32; xq is one token's Q8_K row of
+ * n_blocks super-blocks. */
+int dsx_moe_gate_up_batch(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
+                          const uint8_t *up, const uint8_t *xq, const float *ew,
+                          const int32_t *selected, uint64_t gbpe, uint64_t ubpe, uint32_t n_used,
+                          float clamp, uint32_t n_rows, uint32_t n_blocks);
+/* dispatch::moe_down_batched (crates/v4flash-kernels/src/het/dispatch.rs:121-150):
+ * out[row] = sum_slot down_e[row] . midq[slot]; midq slot-major Q8_K with
+ * xq_slot_stride bytes between slots. */
+int dsx_moe_down_batched(dsx_stream_t stream, int dtype, float *out, const uint8_t *down,
+                         const uint8_t *xq, const int32_t *selected, uint64_t dbpe,
+                         uint32_t xq_slot_stride, uint32_t n_used, uint32_t n_rows,
+                         uint32_t n_blocks_in);
+
+/* ---- by-expert (many tokens) ----------------------------------------------
+ * MoeGroupBuilder::launch + launch_work_items
+ * (crates/v4flash-kernels/src/moe_group_builder.rs:72-130).  One call builds
+ * group_count[n_expert], the exclusive prefix sum group_offset[n_expert+1],
+ * expert_members[b*n_used] = (token << 16) | slot in ascending (token, slot)
+ * order per expert, work_items = (expert << 16) | start in ascending order and
+ * n_work_items[1].  Unlike the reference's atomic builder the order is
+ * deterministic and the member table is compacted (no max_per_expert).
+ * selected entries outside [0, n_expert) are skipped.  b, n_used, n_expert <
+ * 65536; chunk in [1, 16]. */
+int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,
+                        int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
+                        const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
+                        uint32_t chunk);
+/* dispatch::moe_gate_up_chunked_rows (crates/v4flash-kernels/src/het/dispatch.rs:534-570):
+ * mid[b, n_used, n_rows]; xq is [b, n_blocks*292]; ew is [b, n_used].
+ * max_work_items bounds the grid (dispatch::moe_wi_upper_bound, :450-454); the
+ * device-side count is read by the kernel. */
+int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
+                                 const uint8_t *up, const uint8_t *xq, const float *ew,
+                                 const int32_t *group_count, const int32_t *group_offset,
+                                 const int32_t *expert_members, const int32_t *work_items,
+                                 const int32_t *n_work_items, uint32_t max_work_items,
+                                 uint64_t gbpe, uint64_t ubpe, uint32_t n_used, uint32_t chunk,
+                                 float clamp, uint32_t n_rows, uint32_t n_blocks);
+/* dispatch::moe_down_mxfp4 (crates/v4flash-kernels/src/het/dispatch.rs:580-620):
+ * partials[(t*n_used+slot)*n_rows + row] = down_e[row] . midq[t,slot];
+ * midq is [b*n_used] rows of xq_slot_stride bytes. */
+int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, const uint8_t *down,
+                           const uint8_t *xq, const int32_t *group_count,
+                           const int32_t *group_offset, const int32_t *expert_members,
+                           const int32_t *work_items, const int32_t *n_work_items,
+                           uint32_t max_work_items, uint64_t dbpe, uint32_t xq_slot_stride,
+                           uint32_t n_used, uint32_t chunk, uint32_t n_rows,
+                           uint32_t n_blocks_in);
+/* Q2KAccumulateMatvec::launch_reduce_partials (crates/v4flash-kernels/src/q2_k.rs:454-500;
+ * kernels/q2_k_accumulate_matvec_par.hip:714-730): out[t,row] = sum over slots, in
+ * slot order.  selected (nullable): slots with selected < 0 are skipped, so the
+ * caller does not have to zero rows no pick wrote. */
+int dsx_moe_reduce_partials(dsx_stream_t stream, float *out, const float *partials,
+                            const int32_t *selected, uint32_t n_used, uint32_t n_rows, uint32_t b);
+
+/* ---- dense SwiGLU expert (the shared expert) -------------------------------
+ * issue_shared_expert (crates/v4flash-kernels/src/het/forward_layer.rs:3234-;
+ * forward_prefill.rs:3649-3830): out[t,:] (+)= down . Q(swiglu(gate.Q(x), up.Q(x))).
+ * x is f32 [b, hidden]; scratch must hold dsx_dense_ffn_scratch_bytes(). */
+size_t dsx_dense_ffn_scratch_bytes(uint32_t b, uint32_t hidden, uint32_t inter);
+int dsx_dense_ffn(dsx_stream_t stream, int gate_fmt, int up_fmt, int down_fmt, float *out,
+                  const uint8_t *gate, const uint8_t *up, const uint8_t *down, const float *x,
+                  uint32_t b, uint32_t hidden, uint32_t inter, float clamp, int accumulate,
+                  void *scratch);
+
+/* ---- element-wise ----------------------------------------------------------
+ * VecAddInplace::launch (crates/v4flash-kernels/src/ffn.rs:135-153). */
+int dsx_vec_add_inplace(dsx_stream_t stream, float *out, const float *rhs, uint64_t n);
+/* RmsNorm batched (crates/v4flash-kernels/src/rms_norm.rs; kernels/rms_norm.hip:52-). */
+int dsx_rms_norm(dsx_stream_t stream, float *out, const float *x, const float *weight,
+                 uint32_t n, float eps, uint32_t rows);
+/* SwiGluKernel::launch_clamped (crates/v4flash-kernels/src/ffn.rs:36-75). */
+int dsx_swiglu_clamp_weighted(dsx_stream_t stream, float *mid, const float *gate, const float *up,
+                              const float *expert_w, float clamp, uint32_t ff, uint32_t n_experts);
+
+/* ---- weight pipeline ---------------------------------------------------------
+ * Mxfp4Repack (crates/v4flash-kernels/src/mxfp4_repack.rs; kernels/mxfp4_repack.hip:35-65):
+ * HF packed[out, nb*16] + scale[out, nb] -> v2 rows dst[out, nb*17]. nb % 8 == 0. */
+int dsx_mxfp4_repack_hf_to_v2(dsx_stream_t stream, uint8_t *dst, const uint8_t *packed,
+                              const uint8_t *scale, uint32_t out, uint32_t nb);
+/* Dequantize engine rows to f32 (checking aid; crates/v4flash-core/src/kquants.rs:105-111 for
+ * Q8_0, crates/v4flash-kernels/src/mxfp4_tables.rs:38-45 for MXFP4). */
+int dsx_dequant_rows(dsx_stream_t stream, int dtype, float *y, const uint8_t *rows,
+                     uint32_t n_rows, uint32_t cols);
+
+/* ---- the whole layer ---------------------------------------------------------
+ * Modelled on MoeExecutor::run (crates/v4flash-kernels/src/het/remote_experts.rs:7432-7443)
+ * plus the router in front and the shared expert + combine behind it
+ * (forward_prefill.rs:9095-9118, 12227-12232).  The descriptor only records
+ * pointers and dimensions; no weight is copied. */
+typedef struct {
+    uint32_t hidden, inter, n_expert, n_used;
+    int gate_fmt, up_fmt, down_fmt;
+    const uint8_t *gate, *up, *down; /* [n_expert] experts each */
+    uint64_t gate_bpe, up_bpe, down_bpe;
+    float clamp;
+    /* router */
+    uint32_t router_mode, n_group, topk_group;
+    float route_scale, route_eps;
+    const float *bias; /* [n_expert] or NULL */
+    /* shared expert, sh_inter == 0 for none */
+    uint32_t sh_inter;
+    int sh_gate_fmt, sh_up_fmt, sh_down_fmt;
+    const uint8_t *sh_gate, *sh_up, *sh_down;
+    float sh_clamp;
+} dsx_moe_layer_desc;
+
+typedef struct dsx_moe_layer dsx_moe_layer;
+
+int dsx_moe_layer_create(const dsx_moe_layer_desc *desc, dsx_moe_layer **out);
+void dsx_moe_layer_destroy(dsx_moe_layer *layer);
+/* Bytes of caller-provided device scratch for up to max_tokens tokens. */
+size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
+/* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],
+ * logits f32 [n_tokens, n_expert].  selected_out / weights_out (nullable) receive
+ * the routing.  If selected_in is non-NULL the router is skipped and
+ * selected_in / weights_in are used (pinned routing). */
+int dsx_moe_layer_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *out, const float *x,
+                          const float *logits, uint32_t n_tokens, void *workspace,
+                          size_t workspace_bytes, int32_t *selected_out, float *weights_out,
+                          const int32_t *selected_in, const float *weights_in);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

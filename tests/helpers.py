@@ -1,0 +1,139 @@
+"""Shared helpers of the test-suite: synthetic layers on host and device, parity metrics."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+from deepstrix_amd import synth
+from deepstrix_amd.capi import FMT_MXFP4, FMT_Q8_0
+from oracle import ref
+
+ROUTER = {"sqrt_softplus": 0, "sigmoid": 1, "softmax": 2}
+
+
+@dataclass
+class Shape:
+    hidden: int
+    inter: int
+    n_expert: int
+    n_used: int
+    gate_fmt: int = FMT_MXFP4
+    down_fmt: int = FMT_MXFP4
+    shared: bool = True
+    sh_gate_fmt: Optional[int] = None
+    sh_down_fmt: Optional[int] = None
+    clamp: float = 0.0
+    router_mode: int = 1
+    n_group: int = 1
+    topk_group: int = 1
+    route_scale: float = 1.0
+    route_eps: float = 1e-20
+    bias_sigma: float = 0.0
+    seed: int = 0xD5EE0000
+
+    @property
+    def shg(self):
+        return self.sh_gate_fmt if self.sh_gate_fmt is not None else self.gate_fmt
+
+    @property
+    def shd(self):
+        return self.sh_down_fmt if self.sh_down_fmt is not None else self.down_fmt
+
+
+# BASELINE configs
+CFG1 = Shape(2048, 1408, 64, 6, FMT_Q8_0, FMT_Q8_0, router_mode=2, seed=0xD5EE0001)
+CFG2 = Shape(7168, 2048, 256, 8, router_mode=1, n_group=8, topk_group=4, route_scale=2.5,
+             bias_sigma=0.01, seed=0xD5EE0002)
+CFG5 = Shape(7168, 2048, 256, 8, FMT_MXFP4, FMT_Q8_0, router_mode=1, route_scale=2.5,
+             seed=0xD5EE0005)
+
+
+def host_expert(s: Shape, which: int, fmt: int, rows: int, cols: int, e: int) -> np.ndarray:
+    return synth.weights_host(fmt, s.seed, which, rows, cols, first_row=e * rows)
+
+
+def host_weights(s: Shape, experts=None) -> ref.MoeWeights:
+    """Host copy of the layer.  `experts`: generate only these experts' bytes (the others are
+    left zero), to keep large shapes cheap on the CPU."""
+    gb = synth.matrix_bytes(s.gate_fmt, s.inter, s.hidden)
+    db = synth.matrix_bytes(s.down_fmt, s.hidden, s.inter)
+    gate = np.zeros(s.n_expert * gb, np.uint8)
+    up = np.zeros(s.n_expert * gb, np.uint8)
+    down = np.zeros(s.n_expert * db, np.uint8)
+    for e in (range(s.n_expert) if experts is None else sorted(set(int(v) for v in experts))):
+        gate[e * gb:(e + 1) * gb] = host_expert(s, synth.T_GATE, s.gate_fmt, s.inter, s.hidden, e)
+        up[e * gb:(e + 1) * gb] = host_expert(s, synth.T_UP, s.gate_fmt, s.inter, s.hidden, e)
+        down[e * db:(e + 1) * db] = host_expert(s, synth.T_DOWN, s.down_fmt, s.hidden, s.inter, e)
+    w = ref.MoeWeights(s.hidden, s.inter, s.n_expert, s.n_used, gate, up, down, s.gate_fmt,
+                       s.gate_fmt, s.down_fmt, s.clamp)
+    if s.shared:
+        w.sh_inter = s.inter
+        w.sh_gate = host_expert(s, synth.T_SH_GATE, s.shg, s.inter, s.hidden, 0)
+        w.sh_up = host_expert(s, synth.T_SH_UP, s.shg, s.inter, s.hidden, 0)
+        w.sh_down = host_expert(s, synth.T_SH_DOWN, s.shd, s.hidden, s.inter, 0)
+        w.sh_gate_fmt = w.sh_up_fmt = s.shg
+        w.sh_down_fmt = s.shd
+        w.sh_clamp = s.clamp
+    return w
+
+
+def host_inputs(s: Shape, T: int, logit_shift: Optional[np.ndarray] = None):
+    x = synth.normal_host(s.seed, synth.T_X, T * s.hidden).reshape(T, s.hidden)
+    # BASELINE config 2: bf16 activations, converted to f32 exactly
+    x = (x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)
+    logits = synth.normal_host(s.seed, synth.T_LOGITS, T * s.n_expert).reshape(T, s.n_expert)
+    if logit_shift is not None:
+        logits = (logits + logit_shift[None, :]).astype(np.float32)
+    bias = synth.normal_host(s.seed, synth.T_BIAS, s.n_expert, s.bias_sigma) if s.bias_sigma else None
+    return x, logits, bias
+
+
+def device_weights(s: Shape, device="cuda"):
+    """The same layer generated on the GPU (identical bytes)."""
+    import torch
+    from deepstrix_amd.executor import LayerWeights
+    gate = synth.weights_dev(s.gate_fmt, s.seed, synth.T_GATE, s.n_expert * s.inter, s.hidden)
+    up = synth.weights_dev(s.gate_fmt, s.seed, synth.T_UP, s.n_expert * s.inter, s.hidden)
+    down = synth.weights_dev(s.down_fmt, s.seed, synth.T_DOWN, s.n_expert * s.hidden, s.inter)
+    w = LayerWeights(s.hidden, s.inter, s.n_expert, s.n_used, gate, up, down, s.gate_fmt,
+                     s.gate_fmt, s.down_fmt, s.clamp, s.router_mode, s.n_group, s.topk_group,
+                     s.route_scale, s.route_eps)
+    if s.bias_sigma:
+        w.bias = synth.normal_dev(s.seed, synth.T_BIAS, s.n_expert, s.bias_sigma)
+    if s.shared:
+        w.sh_inter = s.inter
+        w.sh_gate = synth.weights_dev(s.shg, s.seed, synth.T_SH_GATE, s.inter, s.hidden)
+        w.sh_up = synth.weights_dev(s.shg, s.seed, synth.T_SH_UP, s.inter, s.hidden)
+        w.sh_down = synth.weights_dev(s.shd, s.seed, synth.T_SH_DOWN, s.hidden, s.inter)
+        w.sh_gate_fmt = w.sh_up_fmt = s.shg
+        w.sh_down_fmt = s.shd
+        w.sh_clamp = s.clamp
+    torch.cuda.synchronize()
+    return w
+
+
+def oracle_route(s: Shape, logits, bias):
+    return ref.router_topk(logits, bias, s.n_used, s.route_scale, s.route_eps, s.router_mode,
+                           s.n_group, s.topk_group)
+
+
+def max_rel(a: np.ndarray, b_ref: np.ndarray) -> float:
+    """max|a - ref| / max|ref| -- the reference's check() metric
+    (crates/v4flash-kernels/tests/mxfp4_pair_oracle.rs:86-100)."""
+    denom = float(np.abs(b_ref).max())
+    return float(np.abs(a.astype(np.float64) - b_ref.astype(np.float64)).max()) / max(denom, 1e-30)
+
+
+def routing_mismatch_explained(sel_gpu, sel_ref, scores, n_used, tol=1e-4):
+    """True when every token whose pick SET differs has a (k-th, (k+1)-th) score gap <= tol."""
+    bad = []
+    for t in range(sel_ref.shape[0]):
+        if set(sel_gpu[t].tolist()) == set(sel_ref[t].tolist()):
+            continue
+        s = np.sort(scores[t][np.isfinite(scores[t])])[::-1]
+        gap = s[n_used - 1] - s[n_used] if s.size > n_used else np.inf
+        if gap > tol:
+            bad.append((t, float(gap)))
+    return bad
