@@ -58,15 +58,20 @@ __device__ __forceinline__ void split_q(int q, uint32_t &hi_byte, uint32_t &lo_b
 // ---------------------------------------------------------------------------------------
 // Staged activation tile in LDS, for one super-block (256 k) and NT token columns.
 //
-// The MFMA's B operand gives lane l column (l % 16) and the 32-k block (l / 16) of a 128-k
-// half, 32 bytes in k order.  The weights' nibble byte j holds element j (low nibble) and
-// element 16 + j (high nibble) of the block, so MFMA position p of a block is element
-// p/2 (p even) or 16 + p/2 (p odd); the activation bytes are stored in that order.
+// Operand layout of the instruction for one 128-k half (measured with one-hot probes):
+//   A, FP4, 4 VGPRs:  lane l holds row l % 16, k = 32 * (l / 16) + n for nibble n = 0..31
+//                     (low nibble of byte 0 first) -- exactly one 16-byte weight block;
+//   B, FP8, 8 VGPRs:  lane l holds column l % 16; bytes 0..15 are k = 16 * (l / 16) + p,
+//                     bytes 16..31 are k = 64 + 16 * (l / 16) + (p - 16).
+// The weights' nibble byte j holds element j (low) and element 16 + j (high) of its block,
+// so nibble n of block b is element n/2 (n even) or 16 + n/2 (n odd) and sits at
+// k = 32 * b + n.  The activation for that k goes to B lane group (k % 64) / 16, byte
+// 16 * (k / 64) + k % 16:
 //
-//   tile[half h][plane][chunk c][kb][column][16 B]     half = block/4, kb = block%4,
-//   plane 0 = high (x16), plane 1 = low, chunk c = positions 16c .. 16c+15.
-// A lane reads its operand as two 16-byte chunks; consecutive lanes read consecutive
-// 16-byte words (NT == 16) or broadcast (NT < 16).
+//   tile[half h][plane][chunk c][kb][column][16 B]    c = k / 64, kb = (k % 64) / 16,
+//   plane 0 = high (x16), plane 1 = low.
+// A lane reads its operand as the two 16-byte chunks c = 0, 1; consecutive lanes read
+// consecutive 16-byte words (NT == 16) or broadcast (NT < 16).
 // ---------------------------------------------------------------------------------------
 template <int NT>
 __device__ __forceinline__ uint32_t tile_off(uint32_t h, uint32_t plane, uint32_t c, uint32_t kb,
@@ -75,8 +80,8 @@ __device__ __forceinline__ uint32_t tile_off(uint32_t h, uint32_t plane, uint32_
 }
 
 // One wave converts one Q8_K block (292 B in global memory) into the tile of column `col`.
-// lane -> (block b32 = lane / 8, dword d = lane % 8); dword d holds positions 4d..4d+3 =
-// elements (2d, 16+2d, 2d+1, 17+2d) of the block.
+// lane -> (block b32 = lane / 8, dword d = lane % 8); dword d holds nibble positions
+// n = 4d..4d+3 = elements (2d, 16+2d, 2d+1, 17+2d) of the block.
 template <int NT>
 __device__ __forceinline__ void stage_q8k_block(uint8_t *tile, float *yd_slot,
                                                 const uint8_t *__restrict__ blk, uint32_t col,
@@ -94,7 +99,8 @@ __device__ __forceinline__ void stage_q8k_block(uint8_t *tile, float *yd_slot,
     split_q(q3, h3, l3);
     const uint32_t hw = h0 | (h1 << 8) | (h2 << 16) | (h3 << 24);
     const uint32_t lw = l0 | (l1 << 8) | (l2 << 16) | (l3 << 24);
-    const uint32_t h = b32 >> 2, kb = b32 & 3u, c = d >> 2, o = (d & 3u) * 4u;
+    const uint32_t h = b32 >> 2, b = b32 & 3u;
+    const uint32_t c = b >> 1, kb = 2u * (b & 1u) + (d >> 2), o = (d & 3u) * 4u;
     *(uint32_t *)(tile + tile_off<NT>(h, 0, c, kb, col) + o) = hw;
     *(uint32_t *)(tile + tile_off<NT>(h, 1, c, kb, col) + o) = lw;
     if (lane == 0) *yd_slot = *(const float *)blk;

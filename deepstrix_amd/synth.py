@@ -45,7 +45,15 @@ def lib() -> C.CDLL:
 
 
 def matrix_bytes(fmt: int, rows: int, cols: int) -> int:
-    return rows * (cols // 256) * 136 if fmt == FMT_MXFP4 else rows * (cols // 32) * 34
+    if fmt == FMT_MXFP4:
+        if cols <= 0 or cols % 256:
+            raise ValueError(f"MXFP4 rows need cols % 256 == 0, got {cols}")
+        return rows * (cols // 256) * 136
+    if fmt == FMT_Q8_0:
+        if cols <= 0 or cols % 32:
+            raise ValueError(f"Q8_0 rows need cols % 32 == 0, got {cols}")
+        return rows * (cols // 32) * 34
+    raise ValueError(f"unknown weight format {fmt}")
 
 
 def normal_host(seed, tensor_id, n, sigma=1.0, mean=0.0, offset=0) -> np.ndarray:

@@ -89,14 +89,15 @@ def test_router_matches_oracle(mode, E, k, ng, tg, scale, eps, bias_sigma):
     assert H.routing_mismatch_explained(sel, rsel, scores, k) == []
     same = np.array([np.array_equal(sel[t], rsel[t]) for t in range(T)])
     assert same.mean() > 0.97
-    assert np.array_equal(sel[0], np.arange(k)) or ng > 1
+    if bias is None and ng <= 1:
+        assert np.array_equal(sel[0], np.arange(k))     # all tied: lowest indices win
     np.testing.assert_allclose(w[same], rw[same], rtol=2e-5, atol=1e-7)
     if ng > 1:
         gs = E // ng
         assert all(len(set((sel[t] // gs).tolist())) <= tg for t in range(T))
 
 
-def small_case(hidden=512, inter=64, E=8, k=3, seed=11):
+def small_case(hidden=512, inter=256, E=8, k=3, seed=11):
     s = H.Shape(hidden, inter, E, k, shared=True, seed=seed, clamp=10.0)
     return s, H.host_weights(s)
 
