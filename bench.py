@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE feed-forward layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload: BASELINE config 2 -- DeepSeek-V3-shape layer (hidden 7168, 256 routed experts + 1
+shared, top-8 sigmoid gating with bias, 8 groups / top-4, scale 2.5, intermediate 2048, MXFP4
+weights, bf16-valued activations) at T = 1.  One step = one layer forward for one token.
+Steps rotate over several independent layers (different weights, different token) so that no
+weight byte is served from the last-level cache: the cold-weight regime of real decoding.
+
+Prints ONE JSON line (metric, value, roofline, cpu_baseline, ...).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E
+MATRIX_BYTES = 7168 * (2048 // 32) * 17   # one MXFP4 7168 x 2048 matrix = 7,798,784 B
+EXPERT_BYTES = 3 * MATRIX_BYTES           # 23,396,352 B
+TOKEN_BYTES = 9 * EXPERT_BYTES            # 8 routed + 1 shared = 210,567,168 B / token
+GATE_UP_BYTES = 9 * 2 * MATRIX_BYTES      # what one gate/up launch streams at T = 1
+
+
+class Hip:
+    """The few HIP runtime calls the harness needs (events on the launch stream)."""
+
+    def __init__(self):
+        self.l = C.CDLL("libamdhip64.so")
+        self.l.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.l.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.l.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.l.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.l.hipEventDestroy.argtypes = [C.c_void_p]
+
+    def event(self):
+        e = C.c_void_p()
+        rc = self.l.hipEventCreate(C.byref(e))
+        if rc:
+            raise RuntimeError(f"hipEventCreate: {rc}")
+        return e
+
+    def elapsed_ms(self, a, b) -> float:
+        ms = C.c_float()
+        rc = self.l.hipEventElapsedTime(C.byref(ms), a, b)
+        if rc:
+            raise RuntimeError(f"hipEventElapsedTime: {rc}")
+        return float(ms.value)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=4, help="independent layers the steps rotate over")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from deepstrix_amd import capi
+    from deepstrix_amd.executor import MoeLayer
+    from tests import helpers as H
+
+    torch.cuda.set_device(0)
+    capi.init()
+    hip = Hip()
+    base = H.CFG2
+    K, W, L = args.steps, args.warmup, args.layers
+    layers, weights = [], []
+    for i in range(L):
+        s = H.Shape(**{**base.__dict__, "seed": base.seed + 0x100 * i})
+        dw = H.device_weights(s)
+        weights.append(dw)
+        layers.append(MoeLayer(dw, 64))
+    # one fresh token per step (bf16-valued activations, N(0,1) logits)
+    n_tok = W + K
+    x_all, lg_all, _ = H.host_inputs(base, n_tok)
+    x_all = torch.from_numpy(x_all).cuda()
+    lg_all = torch.from_numpy(lg_all).cuda()
+    out = torch.empty((1, base.hidden), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step(i):
+        layers[i % L].run(x_all[i:i + 1], lg_all[i:i + 1], out=out)
+
+    for i in range(W):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(W, W + K):
+        step(i)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / K
+
+    # same steps again with events around the dominant kernel (gate/up) and the whole chain
+    evs = [(hip.event(), hip.event(), hip.event(), hip.event()) for _ in range(K)]
+    for j, i in enumerate(range(W, W + K)):
+        a, b, c, d = evs[j]
+        lay = layers[i % L]
+        lay.set_profile_events(b, c, None)
+        hip.l.hipEventRecord(a, stream)
+        step(i)
+        hip.l.hipEventRecord(d, stream)
+    torch.cuda.synchronize()
+    for lay in layers:
+        lay.set_profile_events(None, None, None)
+    gu_ms = np.array([hip.elapsed_ms(b, c) for (_, b, c, _) in evs])
+    chain_ms = np.array([hip.elapsed_ms(a, d) for (a, _, _, d) in evs])
+    gu_avg_us = float(gu_ms.mean() * 1e3)
+    achieved = GATE_UP_BYTES / (gu_avg_us * 1e-6) / 1e9
+
+    # other token counts of the same config (informative)
+    extra = {"gate_up_us_p50": float(np.median(gu_ms) * 1e3),
+             "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
+             "layer_GBps_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9,
+             "layer_frac_of_hbm_peak_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    for T in (4, 16, 64):
+        xs, ls, _ = H.host_inputs(H.Shape(**{**base.__dict__, "seed": base.seed + T}), T)
+        xs, ls = torch.from_numpy(xs).cuda(), torch.from_numpy(ls).cuda()
+        o = torch.empty((T, base.hidden), dtype=torch.float32, device="cuda")
+        reps = 8
+        for r in range(2):
+            layers[r % L].run(xs, ls, out=o)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for r in range(reps):
+            layers[r % L].run(xs, ls, out=o)
+        torch.cuda.synchronize()
+        extra[f"us_per_token_T{T}"] = (time.perf_counter() - t1) * 1e6 / reps / T
+
+    result = {
+        "metric": "moe_layer_us_per_token_T1",
+        "value": ms_per_step * 1e3,
+        "unit": "us/token",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp4 weights x int8 (Q8_K) activations, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: V3-shape MXFP4 MoE layer decode, T=1 "
+                               "(hidden 7168, 256+1 experts, top-8 sigmoid+bias, 8 groups/top-4, "
+                               "scale 2.5, inter 2048); cold weights, steps rotate over "
+                               f"{L} layers", "tokens_per_step": 1, "layers_rotated": L,
+                   "algorithmic_bytes_per_token": TOKEN_BYTES},
+        "roofline": {"bound": "hbm", "kernel": "k_mxfp4_gate_up<1,false> (gate+up+SwiGLU, 8 routed "
+                     "+ 1 shared expert)", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": GATE_UP_BYTES, "avg_launch_us": gu_avg_us},
+        "extra": extra,
+    }
+
+    if not args.no_cpu:
+        # CPU baseline: the oracle (a port of the reference arithmetic) on the host cores,
+        # same layer-0 weights, decode tokens one at a time, bounded by --cpu-seconds.
+        from oracle import ref
+        dw = weights[0]
+        hw = ref.MoeWeights(base.hidden, base.inter, base.n_expert, base.n_used,
+                            dw.gate.cpu().numpy(), dw.up.cpu().numpy(), dw.down.cpu().numpy(),
+                            clamp=base.clamp, sh_inter=base.inter, sh_gate=dw.sh_gate.cpu().numpy(),
+                            sh_up=dw.sh_up.cpu().numpy(), sh_down=dw.sh_down.cpu().numpy())
+        bias = dw.bias.cpu().numpy()
+        xs = x_all[:256].cpu().numpy()
+        ls = lg_all[:256].cpu().numpy()
+        threads = ref.max_threads()
+        done, t1 = 0, time.perf_counter()
+        while done < xs.shape[0] and (time.perf_counter() - t1) < args.cpu_seconds:
+            sel, w = ref.router_topk(ls[done:done + 1], bias, base.n_used, base.route_scale,
+                                     base.route_eps, base.router_mode, base.n_group,
+                                     base.topk_group)
+            ref.moe_forward(hw, xs[done:done + 1], sel, w)
+            done += 1
+        cpu_s = time.perf_counter() - t1
+        result["cpu_baseline"] = {
+            "value": cpu_s * 1e6 / max(done, 1), "unit": "us/token", "cores": threads,
+            "kind": "port",
+            "sample": f"{done} tokens decoded one at a time through the C oracle "
+                      f"(OpenMP, {threads} threads) on layer 0 of the same workload, {cpu_s:.1f} s"}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -87,6 +87,10 @@ class MoeLayer:
             lib().dsx_moe_layer_destroy(h)
             self._h = None
 
+    def set_profile_events(self, gate_up_begin=None, gate_up_end=None, down_end=None):
+        """hipEvent_t handles (ints) recorded around the gate/up launch and after down."""
+        check(lib().dsx_moe_layer_set_profile_events(self._h, gate_up_begin, gate_up_end, down_end))
+
     def run(self, x: torch.Tensor, logits: Optional[torch.Tensor] = None, out=None,
             selected_in=None, weights_in=None, want_routing=False):
         """x f32 [T, hidden], logits f32 [T, n_expert] -> out f32 [T, hidden]."""

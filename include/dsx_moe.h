@@ -204,6 +204,11 @@ typedef struct dsx_moe_layer dsx_moe_layer;
 
 int dsx_moe_layer_create(const dsx_moe_layer_desc *desc, dsx_moe_layer **out);
 void dsx_moe_layer_destroy(dsx_moe_layer *layer);
+/* Measurement aid with no counterpart in the reference: hipEvent_t handles (or NULL) that
+ * dsx_moe_layer_forward records on its stream right before and right after the gate/up
+ * launch and after the down launch, so a harness can time the dominant kernel in place. */
+int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, void *gate_up_end,
+                                     void *down_end);
 /* Bytes of caller-provided device scratch for up to max_tokens tokens. */
 size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
 /* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],
