@@ -49,17 +49,28 @@ void allow_lds(K kernel) {
 std::once_flag g_attr_once;
 void raise_lds_limits() {
     std::call_once(g_attr_once, [] {
-        allow_lds(k_mxfp4_gate_up<1, false>);
-        allow_lds(k_mxfp4_gate_up<1, true>);
-        allow_lds(k_mxfp4_gate_up<2, true>);
-        allow_lds(k_mxfp4_gate_up<4, true>);
-        allow_lds(k_mxfp4_gate_up<8, true>);
-        allow_lds(k_mxfp4_down_decode);
-        allow_lds(k_mxfp4_down_by_expert<1>);
-        allow_lds(k_mxfp4_down_by_expert<2>);
-        allow_lds(k_mxfp4_down_by_expert<4>);
-        allow_lds(k_mxfp4_down_by_expert<8>);
-        allow_lds(k_mxfp4_down_by_expert<16>);
+        allow_lds(k_mxfp4_gate_up<1, false, false, false>);
+        allow_lds(k_mxfp4_gate_up<1, false, true, true>);
+        allow_lds(k_mxfp4_gate_up<1, true, false, false>);
+        allow_lds(k_mxfp4_gate_up<2, true, false, false>);
+        allow_lds(k_mxfp4_gate_up<4, true, false, false>);
+        allow_lds(k_mxfp4_gate_up<8, true, false, false>);
+        allow_lds(k_mxfp4_gate_up<1, true, true, false>);
+        allow_lds(k_mxfp4_gate_up<2, true, true, false>);
+        allow_lds(k_mxfp4_gate_up<4, true, true, false>);
+        allow_lds(k_mxfp4_gate_up<8, true, true, false>);
+        allow_lds(k_mxfp4_down_decode<false>);
+        allow_lds(k_mxfp4_down_decode<true>);
+        allow_lds(k_mxfp4_down_by_expert<1, false>);
+        allow_lds(k_mxfp4_down_by_expert<2, false>);
+        allow_lds(k_mxfp4_down_by_expert<4, false>);
+        allow_lds(k_mxfp4_down_by_expert<8, false>);
+        allow_lds(k_mxfp4_down_by_expert<16, false>);
+        allow_lds(k_mxfp4_down_by_expert<1, true>);
+        allow_lds(k_mxfp4_down_by_expert<2, true>);
+        allow_lds(k_mxfp4_down_by_expert<4, true>);
+        allow_lds(k_mxfp4_down_by_expert<8, true>);
+        allow_lds(k_mxfp4_down_by_expert<16, true>);
         q8_0_raise_lds_limits();
     });
 }
@@ -75,15 +86,25 @@ int pick_nt(uint32_t chunk) {
 }
 
 template <int NT>
-static void launch_gate_up_be(hipStream_t st, const GateUpParams &p, uint32_t max_wi, size_t lds) {
-    hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true>), dim3(p.n_rows / 16, max_wi),
-                       dim3(kGuWaves * 64), lds, st, p);
+static void launch_gate_up_be(hipStream_t st, const GateUpParams &p, uint32_t max_wi, size_t lds,
+                              bool staged) {
+    if (staged)
+        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, true, false>), dim3(p.n_rows / 16, max_wi),
+                           dim3(kGuWaves * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, false, false>), dim3(p.n_rows / 16, max_wi),
+                           dim3(kGuWaves * 64), lds, st, p);
 }
 
 template <int NT>
-static void launch_down_be(hipStream_t st, const DownByExpertParams &p, uint32_t max_wi, size_t lds) {
-    hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT>), dim3(p.n_rows / 16, max_wi),
-                       dim3(kDownBeWaves * 64), lds, st, p);
+static void launch_down_be(hipStream_t st, const DownByExpertParams &p, uint32_t max_wi, size_t lds,
+                           bool staged) {
+    if (staged)
+        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, true>), dim3(p.n_rows / 16, max_wi),
+                           dim3(kDownBeWaves * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, false>), dim3(p.n_rows / 16, max_wi),
+                           dim3(kDownBeWaves * 64), lds, st, p);
 }
 
 }  // namespace
@@ -130,7 +151,7 @@ int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, cons
             return fail(DSX_ERR_SHAPE, "router_topk: n_group=%u topk_group=%u n_expert=%u", n_group,
                         topk_group, n_expert);
     }
-    hipLaunchKernelGGL(k_router_topk, dim3(b), dim3(64), 0, S(stream), selected, weights, logits,
+    hipLaunchKernelGGL(k_router_topk, dim3(b), dim3(kRouterThreads), 0, S(stream), selected, weights, logits,
                        bias, n_expert, n_used, scale, eps, mode, n_group, topk_group);
     return launched("router_topk");
 }
@@ -171,11 +192,14 @@ int dsx_q8_0_quantize_rows(dsx_stream_t stream, uint8_t *out, const float *x, ui
 }
 
 // ---- decode ---------------------------------------------------------------------------
+// staged != 0: xq is a staged row and (midp, counters) receive the fused quantization of mid.
 static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint8_t *gate,
                                const uint8_t *up, const uint8_t *xq, const float *ew,
                                const int32_t *selected, const uint8_t *sh_gate,
                                const uint8_t *sh_up, float sh_clamp, uint64_t gbpe, uint64_t ubpe,
-                               uint32_t n_used, float clamp, uint32_t n_rows, uint32_t n_blocks) {
+                               uint32_t n_used, float clamp, uint32_t n_rows, uint32_t n_blocks,
+                               bool staged = false, uint8_t *midp = nullptr,
+                               int32_t *counters = nullptr) {
     if (n_used == 0 && !sh_gate) return DSX_OK;
     if (!mid || !gate || !up || !xq || !ew || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: null pointer");
@@ -198,10 +222,20 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
     p.mid = mid; p.gate = gate; p.up = up; p.xq = xq; p.ew = ew; p.selected = selected;
     p.sh_gate = sh_gate; p.sh_up = sh_up; p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used;
     p.chunk = 1; p.clamp = clamp; p.sh_clamp = sh_clamp; p.n_rows = n_rows; p.n_blocks = n_blocks;
-    p.xq_row_bytes = n_blocks * kQ8kBytes;
+    p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
     const uint32_t n_slots = n_used + (sh_gate ? 1u : 0u);
-    hipLaunchKernelGGL((k_mxfp4_gate_up<1, false>), dim3(n_rows / 16, n_slots), dim3(kGuWaves * 64),
-                       lds, st, p);
+    if (staged) {
+        if (n_rows % 256 != 0 || !midp || !counters || !aligned(xq, 16))
+            return fail(DSX_ERR_SHAPE, "moe_gate_up_batch: fused mid quantization needs n_rows %% 256 == 0");
+        p.midp = midp;
+        p.counters = counters;
+        p.midp_row_bytes = staged_row_bytes(n_rows / 256);
+        hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, true, true>), dim3(n_rows / 16, n_slots),
+                           dim3(kGuWaves * 64), lds, st, p);
+    } else {
+        hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, false, false>), dim3(n_rows / 16, n_slots),
+                           dim3(kGuWaves * 64), lds, st, p);
+    }
     return launched("moe_gate_up_batch");
 }
 
@@ -216,7 +250,7 @@ int dsx_moe_gate_up_batch(dsx_stream_t stream, int dtype, float *mid, const uint
 static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t *down,
                             const uint8_t *xq, const int32_t *selected, const uint8_t *sh_down,
                             uint64_t dbpe, uint32_t xq_slot_stride, uint32_t n_used,
-                            uint32_t n_rows, uint32_t n_blocks_in) {
+                            uint32_t n_rows, uint32_t n_blocks_in, bool staged = false) {
     if (!out || !down || !xq || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: null pointer");
     if (n_used > DSX_MAX_USED) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_used=%u", n_used);
@@ -228,9 +262,10 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_down_batched: n_rows=%u must be a multiple of 16", n_rows);
     if (n_blocks_in == 0) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_blocks_in=0");
-    if (xq_slot_stride < n_blocks_in * kQ8kBytes || xq_slot_stride % 4)
+    if (xq_slot_stride < n_blocks_in * (staged ? 516u : (uint32_t)kQ8kBytes) ||
+        xq_slot_stride % (staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_down_batched: xq_slot_stride=%u", xq_slot_stride);
-    if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, 4))
+    if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_down_batched: weights must be 8-byte aligned, xq 4-byte");
     const uint32_t n_slots = n_used + (sh_down ? 1u : 0u);
     const size_t units = (size_t)n_slots * n_blocks_in;
@@ -242,7 +277,10 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     p.out = out; p.down = down; p.xq = xq; p.selected = selected; p.sh_down = sh_down;
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.n_slots = n_slots;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
-    hipLaunchKernelGGL(k_mxfp4_down_decode, dim3(n_rows / 16), dim3(kDownWaves * 64), lds, st, p);
+    if (staged)
+        hipLaunchKernelGGL(k_mxfp4_down_decode<true>, dim3(n_rows / 16), dim3(kDownWaves * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL(k_mxfp4_down_decode<false>, dim3(n_rows / 16), dim3(kDownWaves * 64), lds, st, p);
     return launched("moe_down_batched");
 }
 
@@ -273,13 +311,13 @@ int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *grou
     return launched("moe_group_build");
 }
 
-int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
+static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
                                  const uint8_t *up, const uint8_t *xq, const float *ew,
                                  const int32_t *group_count, const int32_t *group_offset,
                                  const int32_t *expert_members, const int32_t *work_items,
                                  const int32_t *n_work_items, uint32_t max_work_items,
                                  uint64_t gbpe, uint64_t ubpe, uint32_t n_used, uint32_t chunk,
-                                 float clamp, uint32_t n_rows, uint32_t n_blocks) {
+                                 float clamp, uint32_t n_rows, uint32_t n_blocks, bool staged) {
     if (max_work_items == 0) return DSX_OK;
     if (!mid || !gate || !up || !xq || !ew || !group_count || !group_offset || !expert_members ||
         !work_items || !n_work_items)
@@ -296,7 +334,7 @@ int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, con
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: n_rows=%u must be a multiple of 16", n_rows);
     if (n_blocks == 0) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: n_blocks=0");
-    if (gbpe % 8 || ubpe % 8 || !aligned(gate, 8) || !aligned(up, 8) || !aligned(xq, 4))
+    if (gbpe % 8 || ubpe % 8 || !aligned(gate, 8) || !aligned(up, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: weights must be 8-byte aligned, xq 4-byte");
     const int nt = pick_nt(chunk);
     const size_t lds = (size_t)n_blocks * 512 * nt + (size_t)n_blocks * nt * 4;
@@ -310,23 +348,37 @@ int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, con
     p.group_count = group_count; p.group_offset = group_offset; p.members = expert_members;
     p.work_items = work_items; p.n_work_items = n_work_items;
     p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used; p.chunk = chunk; p.clamp = clamp;
-    p.n_rows = n_rows; p.n_blocks = n_blocks; p.xq_row_bytes = n_blocks * kQ8kBytes;
+    p.n_rows = n_rows; p.n_blocks = n_blocks;
+    p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
     hipStream_t st = S(stream);
     switch (nt) {
-        case 1: launch_gate_up_be<1>(st, p, max_work_items, lds); break;
-        case 2: launch_gate_up_be<2>(st, p, max_work_items, lds); break;
-        case 4: launch_gate_up_be<4>(st, p, max_work_items, lds); break;
-        default: launch_gate_up_be<8>(st, p, max_work_items, lds); break;
+        case 1: launch_gate_up_be<1>(st, p, max_work_items, lds, staged); break;
+        case 2: launch_gate_up_be<2>(st, p, max_work_items, lds, staged); break;
+        case 4: launch_gate_up_be<4>(st, p, max_work_items, lds, staged); break;
+        default: launch_gate_up_be<8>(st, p, max_work_items, lds, staged); break;
     }
     return launched("moe_gate_up_chunked_rows");
 }
 
-int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, const uint8_t *down,
+int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
+                                 const uint8_t *up, const uint8_t *xq, const float *ew,
+                                 const int32_t *group_count, const int32_t *group_offset,
+                                 const int32_t *expert_members, const int32_t *work_items,
+                                 const int32_t *n_work_items, uint32_t max_work_items,
+                                 uint64_t gbpe, uint64_t ubpe, uint32_t n_used, uint32_t chunk,
+                                 float clamp, uint32_t n_rows, uint32_t n_blocks) {
+    return gate_up_be_impl(stream, dtype, mid, gate, up, xq, ew, group_count, group_offset,
+                           expert_members, work_items, n_work_items, max_work_items, gbpe, ubpe,
+                           n_used, chunk, clamp, n_rows, n_blocks, false);
+}
+
+static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const uint8_t *down,
                            const uint8_t *xq, const int32_t *group_count,
                            const int32_t *group_offset, const int32_t *expert_members,
                            const int32_t *work_items, const int32_t *n_work_items,
                            uint32_t max_work_items, uint64_t dbpe, uint32_t xq_slot_stride,
-                           uint32_t n_used, uint32_t chunk, uint32_t n_rows, uint32_t n_blocks_in) {
+                           uint32_t n_used, uint32_t chunk, uint32_t n_rows, uint32_t n_blocks_in,
+                           bool staged) {
     if (max_work_items == 0) return DSX_OK;
     if (!partials || !down || !xq || !group_count || !group_offset || !expert_members ||
         !work_items || !n_work_items)
@@ -343,9 +395,10 @@ int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, cons
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: n_rows=%u must be a multiple of 16", n_rows);
     if (n_blocks_in == 0) return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: n_blocks_in=0");
-    if (xq_slot_stride < n_blocks_in * kQ8kBytes || xq_slot_stride % 4)
+    if (xq_slot_stride < n_blocks_in * (staged ? 516u : (uint32_t)kQ8kBytes) ||
+        xq_slot_stride % (staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: xq_slot_stride=%u", xq_slot_stride);
-    if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, 4))
+    if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: weights must be 8-byte aligned, xq 4-byte");
     const int nt = pick_nt(chunk);
     const size_t lds = (size_t)n_blocks_in * 512 * nt + (size_t)n_blocks_in * nt * 4;
@@ -361,13 +414,24 @@ int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, cons
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
     hipStream_t st = S(stream);
     switch (nt) {
-        case 1: launch_down_be<1>(st, p, max_work_items, lds); break;
-        case 2: launch_down_be<2>(st, p, max_work_items, lds); break;
-        case 4: launch_down_be<4>(st, p, max_work_items, lds); break;
-        case 8: launch_down_be<8>(st, p, max_work_items, lds); break;
-        default: launch_down_be<16>(st, p, max_work_items, lds); break;
+        case 1: launch_down_be<1>(st, p, max_work_items, lds, staged); break;
+        case 2: launch_down_be<2>(st, p, max_work_items, lds, staged); break;
+        case 4: launch_down_be<4>(st, p, max_work_items, lds, staged); break;
+        case 8: launch_down_be<8>(st, p, max_work_items, lds, staged); break;
+        default: launch_down_be<16>(st, p, max_work_items, lds, staged); break;
     }
     return launched("moe_down_by_expert");
+}
+
+int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, const uint8_t *down,
+                           const uint8_t *xq, const int32_t *group_count,
+                           const int32_t *group_offset, const int32_t *expert_members,
+                           const int32_t *work_items, const int32_t *n_work_items,
+                           uint32_t max_work_items, uint64_t dbpe, uint32_t xq_slot_stride,
+                           uint32_t n_used, uint32_t chunk, uint32_t n_rows, uint32_t n_blocks_in) {
+    return down_be_impl(stream, dtype, partials, down, xq, group_count, group_offset,
+                        expert_members, work_items, n_work_items, max_work_items, dbpe,
+                        xq_slot_stride, n_used, chunk, n_rows, n_blocks_in, false);
 }
 
 static int reduce_impl(hipStream_t st, float *out, const float *partials, const int32_t *selected,

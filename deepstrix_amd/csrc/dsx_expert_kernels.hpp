@@ -2,8 +2,9 @@
 //
 // One workgroup computes a 16-row tile of one expert for up to NT token columns.  The
 // workgroup's waves split the k dimension by super-block (wave w takes super-blocks
-// w, w + W, ...), each accumulating in registers, and the partial sums are added through
-// LDS in wave order, so results do not depend on scheduling.
+// w, w + W, ...), each accumulating in registers with the next two super-blocks' weights
+// already in flight, and the partial sums are added through LDS in wave order, so results
+// do not depend on scheduling.
 //
 // Two ways to name the tokens of a tile:
 //   decode    one token; grid.y = slot; expert = selected[slot]
@@ -13,39 +14,112 @@
 //             `chunk` members (token << 16 | slot) of that expert
 //             (crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:395-564,
 //              mxfp4_matvec.hip:219-427)
+//
+// Two activation formats:
+//   Q8_K rows (the operator ABI)   converted to FP8 planes while they are staged;
+//   staged rows (inside the layer) already FP8 planes, produced once by the quantizer:
+//             [n_sb][512 B tile][n_sb f32 d], copied to LDS with 128-bit loads.
 #pragma once
 
 #include "dsx_device.hpp"
+#include "dsx_quant.hpp"
 
 namespace dsx {
 
 constexpr int kGuWaves = 4;  // waves per gate/up workgroup
 #define DSX_MAX_SLOTS 17     // n_used <= 16 picks + the shared expert
 
+// Bytes of one staged activation row of n_sb super-blocks (16-byte aligned).
+__host__ __device__ inline uint32_t staged_row_bytes(uint32_t n_sb) {
+    return (n_sb * 516u + 15u) & ~15u;
+}
+
+// Copies staged tiles into LDS.  The workgroup's tile list is `n_cols` columns of `nb`
+// tiles each: column j reads the staged row `row(j)`; its tile b lands in LDS tile
+// `lds_base(j) + b`, column `lds_col(j)`.  All threads take part with 128-bit loads, four
+// in flight per thread.
+struct StageDecode {  // one row, one column (the token of a decode step)
+    const uint8_t *base;
+    __device__ __forceinline__ const uint8_t *row(uint32_t) const { return base; }
+    __device__ __forceinline__ uint32_t lds_base(uint32_t) const { return 0u; }
+    __device__ __forceinline__ uint32_t lds_col(uint32_t) const { return 0u; }
+};
+struct StageSlots {  // down, decode: row j = slot j, its tiles at LDS tiles j*nb.., column 0
+    const uint8_t *base;
+    uint32_t stride, nb;
+    __device__ __forceinline__ const uint8_t *row(uint32_t j) const { return base + (uint64_t)j * stride; }
+    __device__ __forceinline__ uint32_t lds_base(uint32_t j) const { return j * nb; }
+    __device__ __forceinline__ uint32_t lds_col(uint32_t) const { return 0u; }
+};
+struct StageMembers {  // by-expert: row j = rows[idx[j]], LDS tiles 0.., column j
+    const uint8_t *base;
+    uint32_t stride;
+    const uint32_t *idx;  // LDS array
+    __device__ __forceinline__ const uint8_t *row(uint32_t j) const { return base + (uint64_t)idx[j] * stride; }
+    __device__ __forceinline__ uint32_t lds_base(uint32_t) const { return 0u; }
+    __device__ __forceinline__ uint32_t lds_col(uint32_t j) const { return j; }
+};
+
+template <int NT, int NTHREADS, typename Src>
+__device__ __forceinline__ void stage_copy(uint8_t *tiles, float *s_yd, uint32_t n_cols, uint32_t nb,
+                                           uint32_t tid, const Src src) {
+    const uint32_t per_col = nb * 32u;          // 16-byte chunks of one row
+    const uint32_t total = n_cols * per_col;
+    auto ld = [&](uint32_t q) -> uint4 {
+        const uint32_t j = q / per_col, c = q - j * per_col;
+        return *(const uint4 *)(src.row(j) + (size_t)c * 16u);
+    };
+    auto st = [&](uint32_t q, const uint4 &v) {
+        const uint32_t j = q / per_col, c = q - j * per_col;
+        const uint32_t t = src.lds_base(j) + (c >> 5);
+        *(uint4 *)(tiles + (size_t)t * 512u * NT + ((c & 31u) * NT + src.lds_col(j)) * 16u) = v;
+    };
+    for (uint32_t q = tid; q < total; q += 4u * NTHREADS) {
+        const uint32_t q1 = q + NTHREADS, q2 = q + 2u * NTHREADS, q3 = q + 3u * NTHREADS;
+        uint4 v0 = ld(q), v1 = {}, v2 = {}, v3 = {};
+        if (q1 < total) v1 = ld(q1);
+        if (q2 < total) v2 = ld(q2);
+        if (q3 < total) v3 = ld(q3);
+        st(q, v0);
+        if (q1 < total) st(q1, v1);
+        if (q2 < total) st(q2, v2);
+        if (q3 < total) st(q3, v3);
+    }
+    for (uint32_t t = tid; t < n_cols * nb; t += NTHREADS) {
+        const uint32_t j = t / nb, b = t - j * nb;
+        s_yd[(src.lds_base(j) + b) * NT + src.lds_col(j)] =
+            *((const float *)(src.row(j) + (size_t)nb * 512u) + b);
+    }
+}
+
 struct GateUpParams {
     float *mid;            // decode: [n_slots, n_rows]; by-expert: [b * n_used, n_rows]
     const uint8_t *gate;   // [n_expert] experts, stride gbpe
     const uint8_t *up;
-    const uint8_t *xq;     // decode: one Q8_K row; by-expert: [b] rows of xq_row_bytes
+    const uint8_t *xq;     // activation rows (Q8_K or staged), xq_row_bytes apart
     const float *ew;       // decode: [n_used]; by-expert: [b * n_used]
     const int32_t *selected;  // decode only: [n_used]
     const uint8_t *sh_gate;   // decode only: extra slot n_used (weight 1), or null
     const uint8_t *sh_up;
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
+    // fused quantization of mid (FUSE_MIDQ): staged rows out + arrival counters
+    uint8_t *midp;
+    int32_t *counters;     // [dest rows * n_rows / 256], zero on entry
     uint64_t gbpe, ubpe;
     uint32_t n_used, chunk;
     float clamp, sh_clamp;
-    uint32_t n_rows, n_blocks, xq_row_bytes;
+    uint32_t n_rows, n_blocks, xq_row_bytes, midp_row_bytes;
 };
 
 // LDS: [n_blocks] tiles of 512 * NT bytes | yd[n_blocks * NT] floats
-template <int NT, bool BY_EXPERT>
+template <int NT, bool BY_EXPERT, bool STAGED, bool FUSE_MIDQ>
 __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[kGuWaves][2][4][64];
     __shared__ int s_dest[NT];
     __shared__ float s_ew[NT];
     __shared__ uint32_t s_tok[NT];
+    __shared__ int s_last[NT];
 
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + (size_t)p.n_blocks * 512u * NT);
@@ -81,6 +155,13 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
             const int e = p.selected[item];
             if (e < 0) {  // empty slot: defined output, nothing to compute
                 if (tid < 16) p.mid[(uint64_t)item * p.n_rows + row0 + tid] = 0.0f;
+                if (FUSE_MIDQ && row0 % 256u == 0u && wave == 0) {
+                    // the slot's staged row must still be defined: zero tile, d = 0
+                    uint8_t *row = p.midp + (uint64_t)item * p.midp_row_bytes;
+                    const uint32_t blk = row0 / 256u;
+                    *(uint2 *)(row + (size_t)blk * 512u + lane * 8u) = make_uint2(0u, 0u);
+                    if (lane == 0) *(float *)(row + (size_t)(p.n_rows / 256u) * 512u + blk * 4u) = 0.0f;
+                }
                 return;
             }
             gate_e = p.gate + (uint64_t)e * p.gbpe;
@@ -98,45 +179,64 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         }
     }
 
-    // ---- first weight loads go out before the activations are staged ----------------
+    // ---- the first two super-blocks of weights go out before anything else -----------
     const uint32_t r = lane & 15u, kb = lane >> 4;
     const uint64_t row_stride = (uint64_t)p.n_blocks * kSuperBytes;
     const uint8_t *grow = gate_e + (uint64_t)(row0 + r) * row_stride;
     const uint8_t *urow = up_e + (uint64_t)(row0 + r) * row_stride;
     uint32_t sb = wave;
-    WSuper g = {}, u = {};
+    WSuper g0 = {}, u0 = {}, g1 = {}, u1 = {};
     if (sb < p.n_blocks) {
-        g = load_wsuper(grow + (uint64_t)sb * kSuperBytes, kb);
-        u = load_wsuper(urow + (uint64_t)sb * kSuperBytes, kb);
+        g0 = load_wsuper(grow + (uint64_t)sb * kSuperBytes, kb);
+        u0 = load_wsuper(urow + (uint64_t)sb * kSuperBytes, kb);
+    }
+    if (sb + kGuWaves < p.n_blocks) {
+        g1 = load_wsuper(grow + (uint64_t)(sb + kGuWaves) * kSuperBytes, kb);
+        u1 = load_wsuper(urow + (uint64_t)(sb + kGuWaves) * kSuperBytes, kb);
     }
 
+    // ---- activations into LDS -----------------------------------------------------------
     if (BY_EXPERT) __syncthreads();  // s_tok visible
-    for (uint32_t pr = wave; pr < cnt * p.n_blocks; pr += kGuWaves) {
-        const uint32_t j = pr / p.n_blocks, b = pr - j * p.n_blocks;
-        const uint32_t tok = BY_EXPERT ? s_tok[j] : 0u;
-        const uint8_t *blk = p.xq + (uint64_t)tok * p.xq_row_bytes + (uint64_t)b * kQ8kBytes;
-        stage_q8k_block<NT>(tiles + (size_t)b * 512u * NT, s_yd + b * NT + j, blk, j, lane);
+    if (STAGED) {
+        if (BY_EXPERT)
+            stage_copy<NT, kGuWaves * 64>(tiles, s_yd, cnt, p.n_blocks, tid,
+                                          StageMembers{p.xq, p.xq_row_bytes, s_tok});
+        else
+            stage_copy<NT, kGuWaves * 64>(tiles, s_yd, 1u, p.n_blocks, tid, StageDecode{p.xq});
+    } else {
+        for (uint32_t pr = wave; pr < cnt * p.n_blocks; pr += kGuWaves) {
+            const uint32_t j = pr / p.n_blocks, b = pr - j * p.n_blocks;
+            const uint32_t tok = BY_EXPERT ? s_tok[j] : 0u;
+            const uint8_t *blk = p.xq + (uint64_t)tok * p.xq_row_bytes + (uint64_t)b * kQ8kBytes;
+            stage_q8k_block<NT>(tiles + (size_t)b * 512u * NT, s_yd + b * NT + j, blk, j, lane);
+        }
     }
     __syncthreads();
 
-    // ---- k loop ---------------------------------------------------------------------
+    // ---- k loop: two super-blocks of weights in flight per matrix ---------------------
     const uint32_t n = lane & 15u;
     const uint32_t col = (n < cnt) ? n : 0u;
     v4f acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
-    for (; sb < p.n_blocks; sb += kGuWaves) {
-        WSuper gn = g, un = u;
-        const uint32_t nsb = sb + kGuWaves;
-        if (nsb < p.n_blocks) {
-            gn = load_wsuper(grow + (uint64_t)nsb * kSuperBytes, kb);
-            un = load_wsuper(urow + (uint64_t)nsb * kSuperBytes, kb);
-        }
-        const uint8_t *tile = tiles + (size_t)sb * 512u * NT;
-        const BSuper bs = load_bsuper<NT>(tile, kb, col);
-        const float yd = s_yd[sb * NT + col];
+    auto compute = [&](uint32_t s, const WSuper &g, const WSuper &u) {
+        const BSuper bs = load_bsuper<NT>(tiles + (size_t)s * 512u * NT, kb, col);
+        const float yd = s_yd[s * NT + col];
         mfma_super(acc_g, g, bs, yd, kb);
         mfma_super(acc_u, u, bs, yd, kb);
-        g = gn;
-        u = un;
+    };
+    while (sb < p.n_blocks) {
+        compute(sb, g0, u0);
+        if (sb + 2 * kGuWaves < p.n_blocks) {
+            g0 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+            u0 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+        }
+        sb += kGuWaves;
+        if (sb >= p.n_blocks) break;
+        compute(sb, g1, u1);
+        if (sb + 2 * kGuWaves < p.n_blocks) {
+            g1 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+            u1 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+        }
+        sb += kGuWaves;
     }
 
     // ---- add the waves' partial sums in wave order, SwiGLU, store --------------------
@@ -158,7 +258,43 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
             gs += s_red[w][0][i][l];
             us += s_red[w][1][i][l];
         }
-        p.mid[(uint64_t)s_dest[j] * p.n_rows + row0 + rr] = swiglu_clamp(gs, us, clamp, s_ew[j]);
+        const float v = swiglu_clamp(gs, us, clamp, s_ew[j]);
+        float *dst = p.mid + (uint64_t)s_dest[j] * p.n_rows + row0 + rr;
+        if (FUSE_MIDQ)  // written through to memory: another XCD's workgroup will read it
+            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            *dst = v;
+    }
+
+    if (FUSE_MIDQ) {
+        // The sixteen row tiles of a 256-row block arrive in any order; the last one to
+        // arrive quantizes the block of mid into the staged format that down reads.
+        // Hand-off between workgroups (possibly on different XCDs, whose L2s are not
+        // coherent with each other): the mid values are stored write-through, each thread
+        // waits for its stores to be acknowledged, the workgroup meets at a barrier and one
+        // thread bumps the device-scope counter; the last arriver reads with loads that
+        // bypass its own L2.  No cache-wide write-back or invalidate is involved.
+        const uint32_t nblk = p.n_rows / 256u, blk = row0 / 256u;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid < cnt) {
+            const int old = __hip_atomic_fetch_add(&p.counters[(uint32_t)s_dest[tid] * nblk + blk], 1,
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last[tid] = (old == 15) ? 1 : 0;
+        }
+        __syncthreads();
+        for (uint32_t j = wave; j < cnt; j += kGuWaves) {
+            if (!s_last[j]) continue;
+            const float *src = p.mid + (uint64_t)s_dest[j] * p.n_rows + (size_t)blk * 256u + lane * 4u;
+            float4 v;
+            v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            uint8_t *row = p.midp + (uint64_t)s_dest[j] * p.midp_row_bytes;
+            quantize_block_to_staged(v, lane, row + (size_t)blk * 512u,
+                                     (float *)(row + (size_t)nblk * 512u) + blk);
+        }
     }
 }
 
@@ -171,7 +307,7 @@ constexpr int kDownWaves = 8;
 struct DownDecodeParams {
     float *out;             // [n_rows]
     const uint8_t *down;    // [n_expert] experts, stride dbpe
-    const uint8_t *xq;      // slot-major Q8_K, xq_slot_stride bytes per slot
+    const uint8_t *xq;      // slot-major activation rows (Q8_K or staged), xq_slot_stride apart
     const int32_t *selected;  // [n_used]
     const uint8_t *sh_down;   // extra slot n_used, or null
     uint64_t dbpe;
@@ -179,22 +315,24 @@ struct DownDecodeParams {
 };
 
 // LDS: [n_slots * n_blocks_in] tiles of 512 bytes | yd[n_slots * n_blocks_in]
+template <bool STAGED>
 __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const DownDecodeParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[kDownWaves][4][64];
     __shared__ int s_sel[DSX_MAX_SLOTS];
 
-    const uint32_t units = p.n_slots * p.n_blocks_in;
+    const uint32_t nb = p.n_blocks_in;
+    const uint32_t units = p.n_slots * nb;
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + (size_t)units * 512u);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t row0 = blockIdx.x * 16u;
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    const uint64_t row_off = (uint64_t)(row0 + r) * p.n_blocks_in * kSuperBytes;
+    const uint64_t row_off = (uint64_t)(row0 + r) * nb * kSuperBytes;
 
     auto unit_ptr = [&](uint32_t un) -> const uint8_t * {
-        const uint32_t slot = un / p.n_blocks_in, b = un - slot * p.n_blocks_in;
+        const uint32_t slot = un / nb, b = un - slot * nb;
         const int e = (slot < p.n_used) ? p.selected[slot] : 0;
         const uint8_t *base = (slot < p.n_used) ? p.down + (uint64_t)(e < 0 ? 0 : e) * p.dbpe
                                                 : p.sh_down;
@@ -202,28 +340,38 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     };
 
     uint32_t un = wave;
-    WSuper w = {};
-    if (un < units) w = load_wsuper(unit_ptr(un), kb);
+    WSuper w0 = {}, w1 = {};
+    if (un < units) w0 = load_wsuper(unit_ptr(un), kb);
+    if (un + kDownWaves < units) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
 
     if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? p.selected[tid] : 0;
-    for (uint32_t pr = wave; pr < units; pr += kDownWaves) {
-        const uint32_t slot = pr / p.n_blocks_in, b = pr - slot * p.n_blocks_in;
-        const uint8_t *blk = p.xq + (uint64_t)slot * p.xq_slot_stride + (uint64_t)b * kQ8kBytes;
-        stage_q8k_block<1>(tiles + (size_t)pr * 512u, s_yd + pr, blk, 0, lane);
+    if (STAGED) {
+        stage_copy<1, kDownWaves * 64>(tiles, s_yd, p.n_slots, nb, tid,
+                                       StageSlots{p.xq, p.xq_slot_stride, nb});
+    } else {
+        for (uint32_t pr = wave; pr < units; pr += kDownWaves) {
+            const uint32_t slot = pr / nb, b = pr - slot * nb;
+            const uint8_t *blk = p.xq + (uint64_t)slot * p.xq_slot_stride + (uint64_t)b * kQ8kBytes;
+            stage_q8k_block<1>(tiles + (size_t)pr * 512u, s_yd + pr, blk, 0, lane);
+        }
     }
     __syncthreads();
 
     v4f acc = {0.f, 0.f, 0.f, 0.f};
-    for (; un < units; un += kDownWaves) {
-        WSuper wn = w;
-        const uint32_t nun = un + kDownWaves;
-        if (nun < units) wn = load_wsuper(unit_ptr(nun), kb);
-        const uint32_t slot = un / p.n_blocks_in;
-        if (s_sel[slot] >= 0) {  // uniform per wave
-            const BSuper bs = load_bsuper<1>(tiles + (size_t)un * 512u, kb, 0);
-            mfma_super(acc, w, bs, s_yd[un], kb);
+    auto compute = [&](uint32_t u, const WSuper &w) {
+        if (s_sel[u / nb] >= 0) {  // uniform per wave
+            const BSuper bs = load_bsuper<1>(tiles + (size_t)u * 512u, kb, 0);
+            mfma_super(acc, w, bs, s_yd[u], kb);
         }
-        w = wn;
+    };
+    while (un < units) {
+        compute(un, w0);
+        if (un + 2 * kDownWaves < units) w0 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
+        un += kDownWaves;
+        if (un >= units) break;
+        compute(un, w1);
+        if (un + 2 * kDownWaves < units) w1 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
+        un += kDownWaves;
     }
 
     s_red[wave][0][lane] = acc.x;
@@ -248,22 +396,23 @@ constexpr int kDownBeWaves = 4;
 struct DownByExpertParams {
     float *partials;
     const uint8_t *down;
-    const uint8_t *xq;  // [b * n_used] rows of xq_slot_stride bytes
+    const uint8_t *xq;  // [b * n_used] activation rows (Q8_K or staged), xq_slot_stride apart
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
     uint64_t dbpe;
     uint32_t xq_slot_stride, n_used, chunk, n_rows, n_blocks_in;
 };
 
 // LDS: [n_blocks_in] tiles of 512 * NT bytes | yd[n_blocks_in * NT]
-template <int NT>
+template <int NT, bool STAGED>
 __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     const DownByExpertParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[kDownBeWaves][4][64];
     __shared__ int s_dest[NT];
 
+    const uint32_t nb = p.n_blocks_in;
     uint8_t *tiles = smem;
-    float *s_yd = (float *)(smem + (size_t)p.n_blocks_in * 512u * NT);
+    float *s_yd = (float *)(smem + (size_t)nb * 512u * NT);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t row0 = blockIdx.x * 16u;
@@ -280,30 +429,40 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     }
 
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    const uint8_t *wrow = p.down + (uint64_t)e * p.dbpe +
-                          (uint64_t)(row0 + r) * p.n_blocks_in * kSuperBytes;
+    const uint8_t *wrow = p.down + (uint64_t)e * p.dbpe + (uint64_t)(row0 + r) * nb * kSuperBytes;
     uint32_t sb = wave;
-    WSuper w = {};
-    if (sb < p.n_blocks_in) w = load_wsuper(wrow + (uint64_t)sb * kSuperBytes, kb);
+    WSuper w0 = {}, w1 = {};
+    if (sb < nb) w0 = load_wsuper(wrow + (uint64_t)sb * kSuperBytes, kb);
+    if (sb + kDownBeWaves < nb) w1 = load_wsuper(wrow + (uint64_t)(sb + kDownBeWaves) * kSuperBytes, kb);
 
     __syncthreads();
-    for (uint32_t pr = wave; pr < cnt * p.n_blocks_in; pr += kDownBeWaves) {
-        const uint32_t j = pr / p.n_blocks_in, b = pr - j * p.n_blocks_in;
-        const uint8_t *blk = p.xq + (uint64_t)s_dest[j] * p.xq_slot_stride + (uint64_t)b * kQ8kBytes;
-        stage_q8k_block<NT>(tiles + (size_t)b * 512u * NT, s_yd + b * NT + j, blk, j, lane);
+    if (STAGED) {
+        stage_copy<NT, kDownBeWaves * 64>(tiles, s_yd, cnt, nb, tid,
+                                          StageMembers{p.xq, p.xq_slot_stride, (const uint32_t *)s_dest});
+    } else {
+        for (uint32_t pr = wave; pr < cnt * nb; pr += kDownBeWaves) {
+            const uint32_t j = pr / nb, b = pr - j * nb;
+            const uint8_t *blk = p.xq + (uint64_t)s_dest[j] * p.xq_slot_stride + (uint64_t)b * kQ8kBytes;
+            stage_q8k_block<NT>(tiles + (size_t)b * 512u * NT, s_yd + b * NT + j, blk, j, lane);
+        }
     }
     __syncthreads();
 
     const uint32_t n = lane & 15u;
     const uint32_t col = (n < cnt) ? n : 0u;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
-    for (; sb < p.n_blocks_in; sb += kDownBeWaves) {
-        WSuper wn = w;
-        const uint32_t nsb = sb + kDownBeWaves;
-        if (nsb < p.n_blocks_in) wn = load_wsuper(wrow + (uint64_t)nsb * kSuperBytes, kb);
-        const BSuper bs = load_bsuper<NT>(tiles + (size_t)sb * 512u * NT, kb, col);
-        mfma_super(acc, w, bs, s_yd[sb * NT + col], kb);
-        w = wn;
+    auto compute = [&](uint32_t s, const WSuper &w) {
+        const BSuper bs = load_bsuper<NT>(tiles + (size_t)s * 512u * NT, kb, col);
+        mfma_super(acc, w, bs, s_yd[s * NT + col], kb);
+    };
+    while (sb < nb) {
+        compute(sb, w0);
+        if (sb + 2 * kDownBeWaves < nb) w0 = load_wsuper(wrow + (uint64_t)(sb + 2 * kDownBeWaves) * kSuperBytes, kb);
+        sb += kDownBeWaves;
+        if (sb >= nb) break;
+        compute(sb, w1);
+        if (sb + 2 * kDownBeWaves < nb) w1 = load_wsuper(wrow + (uint64_t)(sb + 2 * kDownBeWaves) * kSuperBytes, kb);
+        sb += kDownBeWaves;
     }
 
     s_red[wave][0][lane] = acc.x;

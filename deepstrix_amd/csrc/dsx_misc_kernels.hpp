@@ -7,34 +7,12 @@
 #include <stdint.h>
 
 #include "dsx_device.hpp"
+#include "dsx_quant.hpp"
 
 namespace dsx {
 
-// 64-lane butterfly reductions.  Every lane ends with the full result.
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const uint64_t other = __shfl_xor(v, o, 64);
-        v = other > v ? other : v;
-    }
-    return v;
-}
-__device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-__device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-
-// Order-preserving map f32 -> u32 (larger float => larger integer).
-__device__ __forceinline__ uint32_t f32_key(float f) {
-    const uint32_t b = __float_as_uint(f);
-    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-}
+#define DSX_MAX_EXPERTS_K 512
+#define DSX_MAX_USED_K 16
 
 // ---------------------------------------------------------------------------------------
 // Router.  One wave per token; lane l owns experts l, l+64, ...  (n_expert <= 512).
@@ -45,52 +23,64 @@ __device__ __forceinline__ uint32_t f32_key(float f) {
 // crates/v4flash-kernels/kernels/router_topk.hip:32-36,70-131,
 // crates/v4flash-kernels/kernels/laguna_ops.hip:395-451.
 // ---------------------------------------------------------------------------------------
-constexpr int kRouterPerLane = 8;  // 512 / 64
-
 __device__ __forceinline__ float softplus_stable(float x) {
     if (x > 20.0f) return x;
     if (x < -20.0f) return expf(x);
     return log1pf(expf(x));
 }
 
-__global__ __launch_bounds__(64) void k_router_topk(int32_t *__restrict__ selected,
-                                                    float *__restrict__ weights,
-                                                    const float *__restrict__ logits,
-                                                    const float *__restrict__ bias,
-                                                    uint32_t n_expert, uint32_t n_used, float scale,
-                                                    float eps, uint32_t mode, uint32_t n_group,
-                                                    uint32_t topk_group) {
+constexpr int kRouterThreads = 256;
+
+// One workgroup routes one token.  Thread t owns experts t and t + 256.  The top-k is read
+// off each expert's rank (how many experts beat it: larger score, or equal score and lower
+// index), which every thread counts on its own from 64-bit keys (score, ~index) in LDS.
+__device__ __forceinline__ void route_token(int32_t *__restrict__ selected,
+                                            float *__restrict__ weights,
+                                            const float *__restrict__ lg,
+                                            const float *__restrict__ bias, uint32_t n_expert,
+                                            uint32_t n_used, float scale, float eps, uint32_t mode,
+                                            uint32_t n_group, uint32_t topk_group) {
+    __shared__ __attribute__((aligned(16))) uint64_t s_key[512];
     __shared__ float s_score[512];
+    __shared__ float s_red[kRouterThreads / 64];
     __shared__ float s_gscore[64];
     __shared__ int s_keep[64];
+    __shared__ float s_psel[DSX_MAX_USED_K];
+    __shared__ int s_esel[DSX_MAX_USED_K];
 
-    const uint32_t t = blockIdx.x, lane = threadIdx.x;
-    const float *lg = logits + (uint64_t)t * n_expert;
-
-    float p[kRouterPerLane], s[kRouterPerLane];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t nj = (n_expert + kRouterThreads - 1) / kRouterThreads;  // 1 or 2
+    float p[2], s[2];
     float mx = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < kRouterPerLane; j++) {
-        const uint32_t e = lane + 64u * j;
+    for (int j = 0; j < 2; j++) {
+        const uint32_t e = tid + kRouterThreads * j;
         p[j] = (e < n_expert) ? lg[e] : -INFINITY;
         mx = fmaxf(mx, p[j]);
     }
     if (mode == 2u) {  // softmax
         mx = wave_max_f32(mx);
+        if (lane == 0) s_red[wave] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+        __syncthreads();
         float sum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) {
-            const uint32_t e = lane + 64u * j;
+        for (int j = 0; j < 2; j++) {
+            const uint32_t e = tid + kRouterThreads * j;
             p[j] = (e < n_expert) ? expf(p[j] - mx) : 0.0f;
             sum += p[j];
         }
         sum = wave_sum_f32(sum);
+        if (lane == 0) s_red[wave] = sum;
+        __syncthreads();
+        sum = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) p[j] = p[j] / sum;
+        for (int j = 0; j < 2; j++) p[j] = p[j] / sum;
     } else {
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) {
-            const uint32_t e = lane + 64u * j;
+        for (int j = 0; j < 2; j++) {
+            const uint32_t e = tid + kRouterThreads * j;
             if (e < n_expert)
                 p[j] = (mode == 0u) ? sqrtf(softplus_stable(p[j])) : 1.0f / (1.0f + expf(-p[j]));
             else
@@ -98,137 +88,191 @@ __global__ __launch_bounds__(64) void k_router_topk(int32_t *__restrict__ select
         }
     }
 #pragma unroll
-    for (int j = 0; j < kRouterPerLane; j++) {
-        const uint32_t e = lane + 64u * j;
+    for (int j = 0; j < 2; j++) {
+        const uint32_t e = tid + kRouterThreads * j;
         s[j] = (e < n_expert) ? ((bias != nullptr) ? p[j] + bias[e] : p[j]) : -INFINITY;
+    }
+    if (tid < n_used) {
+        s_esel[tid] = -1;
+        s_psel[tid] = 0.0f;
     }
 
     if (n_group > 1u && topk_group < n_group) {
         // group score = sum of the two largest biased scores of the group
-#pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) {
-            const uint32_t e = lane + 64u * j;
-            if (e < n_expert) s_score[e] = s[j];
-        }
-        __syncthreads();
         const uint32_t gs = n_expert / n_group;
-        if (lane < n_group) {
-            float a = -INFINITY, b = -INFINITY;
-            for (uint32_t i = 0; i < gs; i++) {
-                const float v = s_score[lane * gs + i];
-                if (v > a) {
-                    b = a;
-                    a = v;
-                } else if (v > b) {
-                    b = v;
+        const bool butterfly = gs <= 64u && (gs & (gs - 1u)) == 0u;
+        if (butterfly) {
+            // groups are runs of gs consecutive lanes: top-2 by an xor butterfly
+            for (uint32_t j = 0; j < nj; j++) {
+                float a = s[j], b = -INFINITY;
+                for (uint32_t off = 1; off < gs; off <<= 1) {
+                    const float oa = __shfl_xor(a, (int)off, 64), ob = __shfl_xor(b, (int)off, 64);
+                    const float hi = fmaxf(a, oa), lo = fminf(a, oa);
+                    b = fmaxf(lo, fmaxf(b, ob));
+                    a = hi;
                 }
+                const uint32_t e = tid + kRouterThreads * j;
+                if (e < n_expert && (e % gs) == 0u) s_gscore[e / gs] = (gs >= 2u) ? a + b : a;
             }
-            s_gscore[lane] = (gs >= 2u) ? a + b : a;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; j++) s_score[tid + kRouterThreads * j] = s[j];
+            __syncthreads();
+            if (tid < n_group) {
+                float a = -INFINITY, b = -INFINITY;
+                for (uint32_t i = 0; i < gs; i++) {
+                    const float v = s_score[tid * gs + i];
+                    if (v > a) {
+                        b = a;
+                        a = v;
+                    } else if (v > b) {
+                        b = v;
+                    }
+                }
+                s_gscore[tid] = (gs >= 2u) ? a + b : a;
+            }
         }
         __syncthreads();
-        if (lane < n_group) {
-            // rank among groups: better = larger score, ties -> lower index
-            const float mine = s_gscore[lane];
+        if (tid < n_group) {
+            const float mine = s_gscore[tid];
             uint32_t rank = 0;
             for (uint32_t g = 0; g < n_group; g++) {
                 const float o = s_gscore[g];
-                rank += (o > mine || (o == mine && g < lane)) ? 1u : 0u;
+                rank += (o > mine || (o == mine && g < tid)) ? 1u : 0u;
             }
-            s_keep[lane] = rank < topk_group ? 1 : 0;
+            s_keep[tid] = rank < topk_group ? 1 : 0;
         }
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) {
-            const uint32_t e = lane + 64u * j;
+        for (int j = 0; j < 2; j++) {
+            const uint32_t e = tid + kRouterThreads * j;
             if (e < n_expert && !s_keep[e / gs]) s[j] = -INFINITY;
         }
     }
 
-    float sum = 0.0f;
-    float my_p = 0.0f;  // lane k keeps the k-th pick's unbiased p
-    int my_sel = -1;
-    for (uint32_t k = 0; k < n_used; k++) {
-        uint64_t best = 0;
+    uint64_t key[2];
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) {
-            const uint32_t e = lane + 64u * j;
-            if (e < n_expert) {
-                const uint64_t key = ((uint64_t)f32_key(s[j]) << 32) | (uint64_t)(0xFFFFFFFFu - e);
-                best = key > best ? key : best;
-            }
+    for (int j = 0; j < 2; j++) {
+        const uint32_t e = tid + kRouterThreads * j;
+        key[j] = ((uint64_t)f32_key(s[j]) << 32) | (uint64_t)(0xFFFFFFFFu - e);
+        s_key[e] = key[j];
+    }
+    __syncthreads();
+    // rank = number of keys above mine (keys are distinct: they carry the index)
+    uint32_t rank[2] = {0u, 0u};
+    const uint32_t n4 = (n_expert + 3u) / 4u;  // s_key is padded with the keys of -inf
+    if (nj == 1u) {
+        uint32_t r0 = 0;
+        for (uint32_t q = 0; q < n4; q++) {
+            const ulonglong2 a = *(const ulonglong2 *)(s_key + 4u * q);
+            const ulonglong2 b = *(const ulonglong2 *)(s_key + 4u * q + 2u);
+            r0 += (a.x > key[0]) ? 1u : 0u;
+            r0 += (a.y > key[0]) ? 1u : 0u;
+            r0 += (b.x > key[0]) ? 1u : 0u;
+            r0 += (b.y > key[0]) ? 1u : 0u;
         }
-        best = wave_max_u64(best);
-        // nothing left above -inf: an empty pick (p = 0), as a scan with `>` would leave it
-        const bool none = (uint32_t)(best >> 32) <= f32_key(-INFINITY);
-        const uint32_t e_win = 0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFu);
-        const uint32_t owner = e_win & 63u, jj = e_win >> 6;
-        float pw = 0.0f;
-#pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++) {
-            if ((uint32_t)j == jj) {
-                pw = p[j];
-                if (lane == owner && !none) s[j] = -INFINITY;
-            }
+        rank[0] = r0;
+    } else {
+        uint32_t r0 = 0, r1 = 0;
+        for (uint32_t q = 0; q < n4; q++) {
+            const ulonglong2 a = *(const ulonglong2 *)(s_key + 4u * q);
+            const ulonglong2 b = *(const ulonglong2 *)(s_key + 4u * q + 2u);
+            r0 += (a.x > key[0]) ? 1u : 0u;
+            r0 += (a.y > key[0]) ? 1u : 0u;
+            r0 += (b.x > key[0]) ? 1u : 0u;
+            r0 += (b.y > key[0]) ? 1u : 0u;
+            r1 += (a.x > key[1]) ? 1u : 0u;
+            r1 += (a.y > key[1]) ? 1u : 0u;
+            r1 += (b.x > key[1]) ? 1u : 0u;
+            r1 += (b.y > key[1]) ? 1u : 0u;
         }
-        pw = none ? 0.0f : __shfl(pw, (int)owner, 64);
-        sum += pw;  // every lane adds the same values in pick order
-        if (lane == k) {
-            my_p = pw;
-            my_sel = none ? -1 : (int)e_win;
+        rank[0] = r0;
+        rank[1] = r1;
+    }
+    for (uint32_t j = 0; j < nj; j++) {
+        const uint32_t e = tid + kRouterThreads * j;
+        // an expert masked to -inf is never picked (a scan with `>` from -inf skips it)
+        if (e < n_expert && rank[j] < n_used && s[j] > -INFINITY) {
+            s_esel[rank[j]] = (int)e;
+            s_psel[rank[j]] = p[j];
         }
     }
-    if (sum < eps) sum = eps;
-    if (lane < n_used) {
-        selected[(uint64_t)t * n_used + lane] = my_sel;
-        weights[(uint64_t)t * n_used + lane] = my_p / sum * scale;
+    __syncthreads();
+    if (tid < n_used) {
+        float sum = 0.0f;
+        for (uint32_t k = 0; k < n_used; k++) sum += s_psel[k];  // pick order, as the reference
+        if (sum < eps) sum = eps;
+        selected[tid] = s_esel[tid];
+        weights[tid] = s_psel[tid] / sum * scale;
     }
+}
+
+__global__ __launch_bounds__(kRouterThreads) void k_router_topk(
+    int32_t *__restrict__ selected, float *__restrict__ weights, const float *__restrict__ logits,
+    const float *__restrict__ bias, uint32_t n_expert, uint32_t n_used, float scale, float eps,
+    uint32_t mode, uint32_t n_group, uint32_t topk_group) {
+    const uint32_t t = blockIdx.x;
+    route_token(selected + (uint64_t)t * n_used, weights + (uint64_t)t * n_used,
+                logits + (uint64_t)t * n_expert, bias, n_expert, n_used, scale, eps, mode, n_group,
+                topk_group);
+}
+
+// Front of the layer in one launch: workgroups [0, n_tokens) route one token each (skipped
+// when routing is pinned), the rest quantize the activations into staged rows (one wave per
+// 256-element block) and clear the arrival counters of the fused mid quantization.
+struct FrontParams {
+    int32_t *selected;
+    float *weights;
+    const float *logits;
+    const float *bias;
+    uint8_t *xp;        // staged rows out, xp_row_bytes apart
+    const float *x;     // [n_tokens, k]
+    int32_t *counters;  // n_counters ints to clear (may be null)
+    uint32_t n_expert, n_used;
+    float scale, eps;
+    uint32_t mode, n_group, topk_group;
+    uint32_t n_tokens, n_sb, xp_row_bytes, n_counters, route;
+};
+
+__global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParams p) {
+    const uint32_t n_route = p.route ? p.n_tokens : 0u;
+    if (blockIdx.x < n_route) {
+        const uint32_t t = blockIdx.x;
+        route_token(p.selected + (uint64_t)t * p.n_used, p.weights + (uint64_t)t * p.n_used,
+                    p.logits + (uint64_t)t * p.n_expert, p.bias, p.n_expert, p.n_used, p.scale,
+                    p.eps, p.mode, p.n_group, p.topk_group);
+        return;
+    }
+    const uint32_t qb = blockIdx.x - n_route;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    for (uint32_t i = qb * kRouterThreads + tid; i < p.n_counters; i += (gridDim.x - n_route) * kRouterThreads)
+        p.counters[i] = 0;
+    const uint32_t blk = qb * 4u + (tid >> 6);
+    if (blk >= p.n_tokens * p.n_sb) return;
+    const uint32_t t = blk / p.n_sb, b = blk - t * p.n_sb;
+    const float4 v = *(const float4 *)(p.x + (uint64_t)t * p.n_sb * 256u + (size_t)b * 256u + lane * 4u);
+    uint8_t *row = p.xp + (uint64_t)t * p.xp_row_bytes;
+    quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
+}
+
+// Rows of f32 -> staged rows (the mid activations of the by-expert path).
+__global__ __launch_bounds__(256) void k_quantize_staged(uint8_t *__restrict__ out,
+                                                         const float *__restrict__ x,
+                                                         uint32_t n_rows, uint32_t n_sb,
+                                                         uint32_t row_bytes) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t blk = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (blk >= n_rows * n_sb) return;
+    const uint32_t t = blk / n_sb, b = blk - t * n_sb;
+    const float4 v = *(const float4 *)(x + (uint64_t)blk * 256u + lane * 4u);
+    uint8_t *row = out + (uint64_t)t * row_bytes;
+    quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)n_sb * 512u) + b);
 }
 
 // ---------------------------------------------------------------------------------------
 // Q8_K quantizer: one wave per 256-element block, 4 consecutive elements per lane.
 // crates/v4flash-kernels/kernels/q8_k_quantize.hip:23-90
 // ---------------------------------------------------------------------------------------
-struct Q8kQuant {
-    float d;       // 1 / iscale (0 for an all-zero block)
-    int q[4];      // the lane's four quantized values
-};
-
-__device__ __forceinline__ Q8kQuant q8k_quantize_lane(float4 v, uint32_t lane) {
-    // key = (|x| bits, 255 - index): the largest |x| wins, the first one on ties
-    const float xs[4] = {v.x, v.y, v.z, v.w};
-    uint64_t best = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t idx = lane * 4u + i;
-        const uint64_t key = ((uint64_t)(__float_as_uint(xs[i]) & 0x7FFFFFFFu) << 32) | (255u - idx);
-        best = key > best ? key : best;
-    }
-    best = wave_max_u64(best);
-    const uint32_t amax_bits = (uint32_t)(best >> 32);
-    const uint32_t idx = 255u - (uint32_t)(best & 0xFFu);
-    float cand = xs[0];
-    if ((idx & 3u) == 1u) cand = xs[1];
-    if ((idx & 3u) == 2u) cand = xs[2];
-    if ((idx & 3u) == 3u) cand = xs[3];
-    const float mxv = __shfl(cand, (int)(idx >> 2), 64);
-    Q8kQuant r;
-    if (amax_bits == 0u) {
-        r.d = 0.0f;
-        r.q[0] = r.q[1] = r.q[2] = r.q[3] = 0;
-        return r;
-    }
-    const float iscale = -127.0f / mxv;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        int q = (int)rintf(iscale * xs[i]);
-        q = q > 127 ? 127 : q;
-        q = q < -128 ? -128 : q;
-        r.q[i] = q;
-    }
-    r.d = 1.0f / iscale;
-    return r;
-}
-
 __global__ __launch_bounds__(256) void k_q8k_quantize(uint8_t *__restrict__ out,
                                                       const float *__restrict__ x,
                                                       uint32_t n_blocks) {
@@ -288,7 +332,6 @@ __global__ __launch_bounds__(256) void k_q8_0_quantize(int8_t *__restrict__ xq,
 // moe_work_items_builder.hip:26-44 (atomic order, dense [n_expert x max] table).
 // ---------------------------------------------------------------------------------------
 constexpr int kGbThreads = 1024;
-#define DSX_MAX_EXPERTS_K 512
 
 __global__ __launch_bounds__(kGbThreads) void k_group_build(
     int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,

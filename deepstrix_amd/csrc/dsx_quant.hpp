@@ -1,0 +1,116 @@
+// dsx_quant.hpp -- wave-level Q8_K quantization (one wave per 256-element block) and the
+// "staged" activation format the expert kernels copy straight into LDS.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dsx_device.hpp"
+
+namespace dsx {
+
+// 64-lane butterfly reductions.  Every lane ends with the full result.
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint64_t other = __shfl_xor(v, o, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Order-preserving map f32 -> u32 (larger float => larger integer).
+__device__ __forceinline__ uint32_t f32_key(float f) {
+    const uint32_t b = __float_as_uint(f);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// Q8_K quantizer: one wave per 256-element block, 4 consecutive elements per lane.
+// crates/v4flash-kernels/kernels/q8_k_quantize.hip:23-90
+struct Q8kQuant {
+    float d;       // 1 / iscale (0 for an all-zero block)
+    int q[4];      // the lane's four quantized values
+};
+
+__device__ __forceinline__ Q8kQuant q8k_quantize_lane(float4 v, uint32_t lane) {
+    // key = (|x| bits, 255 - index): the largest |x| wins, the first one on ties
+    const float xs[4] = {v.x, v.y, v.z, v.w};
+    uint64_t best = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t idx = lane * 4u + i;
+        const uint64_t key = ((uint64_t)(__float_as_uint(xs[i]) & 0x7FFFFFFFu) << 32) | (255u - idx);
+        best = key > best ? key : best;
+    }
+    best = wave_max_u64(best);
+    const uint32_t amax_bits = (uint32_t)(best >> 32);
+    const uint32_t idx = 255u - (uint32_t)(best & 0xFFu);
+    float cand = xs[0];
+    if ((idx & 3u) == 1u) cand = xs[1];
+    if ((idx & 3u) == 2u) cand = xs[2];
+    if ((idx & 3u) == 3u) cand = xs[3];
+    const float mxv = __shfl(cand, (int)(idx >> 2), 64);
+    Q8kQuant r;
+    if (amax_bits == 0u) {
+        r.d = 0.0f;
+        r.q[0] = r.q[1] = r.q[2] = r.q[3] = 0;
+        return r;
+    }
+    const float iscale = -127.0f / mxv;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int q = (int)rintf(iscale * xs[i]);
+        q = q > 127 ? 127 : q;
+        q = q < -128 ? -128 : q;
+        r.q[i] = q;
+    }
+    r.d = 1.0f / iscale;
+    return r;
+}
+
+// Quantizes one 256-element block exactly as Q8_K does and writes it in the staged format:
+// a 512-byte tile of FP8 planes (layout of tile_off<1>) and the block scale d.  The int8
+// values never reach memory; they are split as described in dsx_device.hpp.
+// Lane l holds elements 4l..4l+3 of the block, i.e. elements 4m..4m+3 (m = l % 8) of the
+// 32-element block l / 8.  A tile dword holds nibble positions 4d..4d+3 = elements
+// (2d, 16+2d, 2d+1, 17+2d): lanes m and m + 4 of a block exchange their values and build
+// dwords d = 2(m % 4) and 2(m % 4) + 1.
+__device__ __forceinline__ void quantize_block_to_staged(float4 v, uint32_t lane, uint8_t *tile,
+                                                         float *d_out) {
+    const Q8kQuant r = q8k_quantize_lane(v, lane);
+    const uint32_t mine = (uint32_t)(r.q[0] & 0xFF) | ((uint32_t)(r.q[1] & 0xFF) << 8) |
+                          ((uint32_t)(r.q[2] & 0xFF) << 16) | ((uint32_t)(r.q[3] & 0xFF) << 24);
+    const uint32_t other = (uint32_t)__shfl_xor((int)mine, 4, 64);
+    const uint32_t m = lane & 7u;
+    const bool low_half = m < 4u;                   // holds elements < 16 of the block
+    const uint32_t lo4 = low_half ? mine : other;   // elements 4mm .. 4mm+3
+    const uint32_t hi4 = low_half ? other : mine;   // elements 16+4mm .. 16+4mm+3
+    const uint32_t sh = low_half ? 0u : 16u;        // low-half lane: first two; other: last two
+    const int qa = (int8_t)((lo4 >> sh) & 0xFF), qc = (int8_t)((lo4 >> (sh + 8u)) & 0xFF);
+    const int qb = (int8_t)((hi4 >> sh) & 0xFF), qd = (int8_t)((hi4 >> (sh + 8u)) & 0xFF);
+    uint32_t h0, l0, h1, l1, h2, l2, h3, l3;
+    split_q(qa, h0, l0);
+    split_q(qb, h1, l1);
+    split_q(qc, h2, l2);
+    split_q(qd, h3, l3);
+    const uint32_t hw = h0 | (h1 << 8) | (h2 << 16) | (h3 << 24);
+    const uint32_t lw = l0 | (l1 << 8) | (l2 << 16) | (l3 << 24);
+    const uint32_t b32 = lane >> 3, d = 2u * (m & 3u) + (low_half ? 0u : 1u);
+    const uint32_t h = b32 >> 2, b = b32 & 3u;
+    const uint32_t c = b >> 1, kb = 2u * (b & 1u) + (d >> 2), o = (d & 3u) * 4u;
+    *(uint32_t *)(tile + tile_off<1>(h, 0, c, kb, 0) + o) = hw;
+    *(uint32_t *)(tile + tile_off<1>(h, 1, c, kb, 0) + o) = lw;
+    if (lane == 0) *d_out = r.d;
+}
+
+}  // namespace dsx
