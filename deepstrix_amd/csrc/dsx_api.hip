@@ -20,6 +20,7 @@ using namespace dsx;
 namespace {
 
 thread_local char g_err[512] = "";
+int g_num_cu = 256;  // refreshed by dsx_init
 
 int fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -130,6 +131,7 @@ int dsx_init(void) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(DSX_ERR_DEVICE, "dsx_init: device %d is %s; this library is built for gfx950",
                     dev, prop.gcnArchName);
+    g_num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     raise_lds_limits();
     return DSX_OK;
 }

@@ -36,6 +36,31 @@ struct __attribute__((packed, aligned(4))) U2A4 {
     uint32_t x, y;
 };
 
+// Loads that are known to hit global memory.  A pointer that went through LDS or a select is
+// "generic" to the compiler, which then emits flat loads; those count against both memory
+// counters and force a full wait before every use.  Going through address space 1 keeps
+// them global loads whose completion order the compiler can track.
+#define DSX_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef u32x4_t u32x4_a8_t __attribute__((aligned(8)));
+typedef u32x2_t u32x2_a4_t __attribute__((aligned(4)));
+__device__ __forceinline__ U4A8 gload16(const uint8_t *p) {
+    const u32x4_t v = *(const DSX_GLOBAL u32x4_a8_t *)(uintptr_t)p;
+    U4A8 r;
+    r.x = v.x; r.y = v.y; r.z = v.z; r.w = v.w;
+    return r;
+}
+__device__ __forceinline__ U2A4 gload8(const uint8_t *p) {
+    const u32x2_t v = *(const DSX_GLOBAL u32x2_a4_t *)(uintptr_t)p;
+    U2A4 r;
+    r.x = v.x; r.y = v.y;
+    return r;
+}
+__device__ __forceinline__ uint32_t gload4(const uint8_t *p) {
+    return *(const DSX_GLOBAL uint32_t *)(uintptr_t)p;
+}
+
 // E4M3 (OCP) byte of a small non-negative integer m in [0, 15].
 __device__ __forceinline__ uint32_t e4m3_of_uint(uint32_t m) {
     // 0,1,2,3,4,5,6,7 -> 0x00,0x38,0x40,0x44,0x48,0x4A,0x4C,0x4E ; 8..15 -> 0x50 | (m & 7)
@@ -115,9 +140,9 @@ struct WSuper {
 
 __device__ __forceinline__ WSuper load_wsuper(const uint8_t *__restrict__ row_super, uint32_t kb) {
     WSuper w;
-    w.a0 = *(const U4A8 *)(row_super + kb * 16u);
-    w.a1 = *(const U4A8 *)(row_super + 64u + kb * 16u);
-    w.s = *(const U2A4 *)(row_super + 128u);
+    w.a0 = gload16(row_super + kb * 16u);
+    w.a1 = gload16(row_super + 64u + kb * 16u);
+    w.s = gload8(row_super + 128u);
     return w;
 }
 

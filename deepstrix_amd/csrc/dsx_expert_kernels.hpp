@@ -339,10 +339,14 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
         return base + row_off + (uint64_t)b * kSuperBytes;
     };
 
+    // five (slot, super-block) units of weights in flight per wave
     uint32_t un = wave;
-    WSuper w0 = {}, w1 = {};
+    WSuper w0 = {}, w1 = {}, w2 = {}, w3 = {}, w4 = {};
     if (un < units) w0 = load_wsuper(unit_ptr(un), kb);
     if (un + kDownWaves < units) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
+    if (un + 2 * kDownWaves < units) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
+    if (un + 3 * kDownWaves < units) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
+    if (un + 4 * kDownWaves < units) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
 
     if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? p.selected[tid] : 0;
     if (STAGED) {
@@ -364,15 +368,19 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
             mfma_super(acc, w, bs, s_yd[u], kb);
         }
     };
+#define DSX_DOWN_STEP(W)                                                                     \
+    compute(un, W);                                                                          \
+    if (un + 5 * kDownWaves < units) W = load_wsuper(unit_ptr(un + 5 * kDownWaves), kb);     \
+    un += kDownWaves;                                                                        \
+    if (un >= units) break;
     while (un < units) {
-        compute(un, w0);
-        if (un + 2 * kDownWaves < units) w0 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
-        un += kDownWaves;
-        if (un >= units) break;
-        compute(un, w1);
-        if (un + 2 * kDownWaves < units) w1 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
-        un += kDownWaves;
+        DSX_DOWN_STEP(w0)
+        DSX_DOWN_STEP(w1)
+        DSX_DOWN_STEP(w2)
+        DSX_DOWN_STEP(w3)
+        DSX_DOWN_STEP(w4)
     }
+#undef DSX_DOWN_STEP
 
     s_red[wave][0][lane] = acc.x;
     s_red[wave][1][lane] = acc.y;
