@@ -1,0 +1,143 @@
+"""The C-ABI library: loads, exports what the header declares, validates arguments on the
+host before anything is launched (CPU only; no kernel runs here)."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+from deepstrix_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "dsx_moe.h")
+
+
+def declared_functions():
+    """name -> parameter count, parsed from the header's prototypes."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    out = {}
+    for m in re.finditer(r"\b(dsx_[a-z0-9_]+)\s*\(([^;{}]*?)\)\s*;", text, flags=re.S):
+        name, args = m.group(1), m.group(2).strip()
+        out[name] = 0 if args in ("", "void") else args.count(",") + 1
+    return out
+
+
+def test_header_is_plain_c():
+    res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", HEADER],
+                         capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+
+
+def test_library_exports_every_declared_symbol():
+    decl = declared_functions()
+    assert len(decl) >= 25
+    raw = C.CDLL(capi.LIB_PATH)
+    missing = [n for n in decl if not hasattr(raw, n)]
+    assert not missing, f"declared in include/dsx_moe.h but not exported: {missing}"
+
+
+def test_binding_table_matches_the_header():
+    decl = declared_functions()
+    assert set(decl) == set(capi.SIGNATURES), set(decl) ^ set(capi.SIGNATURES)
+    for name, n in decl.items():
+        assert len(capi.SIGNATURES[name][1]) == n, name
+
+
+def test_abi_version_and_constants():
+    text = open(HEADER).read()
+    ver = int(re.search(r"#define\s+DSX_ABI_VERSION\s+(\d+)", text).group(1))
+    assert capi.lib().dsx_abi_version() == ver
+    for cname, val in [("DSX_FMT_Q8_0", capi.FMT_Q8_0), ("DSX_FMT_MXFP4", capi.FMT_MXFP4),
+                       ("DSX_ERR_INVALID_ARG", capi.ERR_INVALID_ARG), ("DSX_ERR_SHAPE", capi.ERR_SHAPE),
+                       ("DSX_ERR_UNSUPPORTED", capi.ERR_UNSUPPORTED), ("DSX_ERR_DEVICE", capi.ERR_DEVICE)]:
+        m = re.search(rf"#define\s+{cname}\s+\(?(-?\d+)\)?", text)
+        assert m and int(m.group(1)) == val, cname
+
+
+def test_layer_desc_struct_matches_the_header_field_order():
+    text = open(HEADER).read()
+    body = re.search(r"typedef struct\s*\{((?:(?!typedef).)*?)\}\s*dsx_moe_layer_desc;", text, flags=re.S)
+    assert body, "dsx_moe_layer_desc not found"
+    src = re.sub(r"/\*.*?\*/", "", body.group(1), flags=re.S)
+    names = []
+    for stmt in src.split(";"):
+        stmt = stmt.strip()
+        if not stmt:
+            continue
+        for part in stmt.split(","):
+            names.append(re.findall(r"[A-Za-z_][A-Za-z0-9_]*", part)[-1])
+    assert names == [f[0] for f in capi.LayerDesc._fields_]
+
+
+def _desc(**kw):
+    d = capi.LayerDesc()
+    d.hidden, d.inter, d.n_expert, d.n_used = 512, 256, 8, 2
+    d.gate_fmt = d.up_fmt = d.down_fmt = capi.FMT_MXFP4
+    d.gate = d.up = d.down = 0x1000  # never dereferenced by create()
+    d.router_mode = capi.ROUTER_SIGMOID
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def _create(d):
+    h = C.c_void_p()
+    rc = capi.lib().dsx_moe_layer_create(C.byref(d), C.byref(h))
+    return rc, h
+
+
+def test_layer_create_validates_before_anything_touches_a_device():
+    l = capi.lib()
+    rc, h = _create(_desc())
+    assert rc == 0 and h.value
+    assert l.dsx_moe_layer_workspace_bytes(h, 4) > l.dsx_moe_layer_workspace_bytes(h, 1) > 0
+    l.dsx_moe_layer_destroy(h)
+
+    cases = [
+        (dict(gate=None), capi.ERR_INVALID_ARG),
+        (dict(n_used=0), capi.ERR_INVALID_ARG),
+        (dict(n_used=9), capi.ERR_INVALID_ARG),            # more picks than experts
+        (dict(hidden=520), capi.ERR_SHAPE),                # not a multiple of 256
+        (dict(inter=96), capi.ERR_SHAPE),                  # MXFP4 down needs inter % 256 == 0
+        (dict(up_fmt=capi.FMT_Q8_0), capi.ERR_UNSUPPORTED),
+        (dict(gate_fmt=12, up_fmt=12), capi.ERR_SHAPE),    # a format id with no layout
+        (dict(sh_inter=256), capi.ERR_INVALID_ARG),        # shared expert without weights
+        (dict(router_mode=3), capi.ERR_INVALID_ARG),
+    ]
+    for kw, code in cases:
+        rc, h = _create(_desc(**kw))
+        assert rc == code, (kw, rc)
+        assert not h.value
+        assert l.dsx_last_error(), kw
+    with pytest.raises(capi.DsxError) as ei:
+        capi.check(_create(_desc(hidden=520))[0])
+    assert ei.value.code == capi.ERR_SHAPE and "hidden=520" in ei.value.message
+
+
+def test_null_layer_handles_are_errors():
+    l = capi.lib()
+    assert l.dsx_moe_layer_set_profile_events(None, None, None, None) == capi.ERR_INVALID_ARG
+    assert l.dsx_moe_layer_workspace_bytes(None, 1) == 0
+    l.dsx_moe_layer_destroy(None)  # a no-op, like free(NULL)
+
+
+def test_missing_library_is_an_import_error_not_a_fallback(monkeypatch):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", os.path.join(ROOT, "deepstrix_amd", "lib", "absent.so"))
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        capi.lib()
+
+
+def test_the_package_never_reaches_into_the_oracle():
+    pkg = os.path.join(ROOT, "deepstrix_amd")
+    offenders = []
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".inc", ".h")):
+                text = open(os.path.join(dirpath, f), errors="replace").read()
+                if re.search(r"\boracle\b|dsx_ref_|libdsx_oracle", text):
+                    offenders.append(f)
+    assert not offenders, offenders
