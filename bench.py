@@ -26,6 +26,12 @@ MATRIX_BYTES = 7168 * (2048 // 32) * 17   # one MXFP4 7168 x 2048 matrix = 7,798
 EXPERT_BYTES = 3 * MATRIX_BYTES           # 23,396,352 B
 TOKEN_BYTES = 9 * EXPERT_BYTES            # 8 routed + 1 shared = 210,567,168 B / token
 GATE_UP_BYTES = 9 * 2 * MATRIX_BYTES      # what one gate/up launch streams at T = 1
+COPY_BYTES = 256 << 20                    # size of the calibration copy (read 256 MiB, write 256 MiB)
+
+# HBM bytes one gate/up launch moves, from hardware counters (two `rocprofv3 --pmc` runs of
+# this script: FETCH_SIZE, then WRITE_SIZE; summary under profiles/).  Each counter is scaled
+# by what it reads for the calibration copy below, whose traffic is known.  None = not measured.
+GATE_UP_TRAFFIC_BYTES = 144_987_136
 
 
 class Hip:
@@ -61,7 +67,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=4, help="independent layers the steps rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path "
@@ -123,6 +129,15 @@ def main():
     gu_avg_us = float(gu_ms.mean() * 1e3)
     achieved = GATE_UP_BYTES / (gu_avg_us * 1e-6) / 1e9
 
+    # a copy of known size, so that byte counters collected over this run can be scaled
+    from deepstrix_amd import synth
+    c_src = torch.empty(COPY_BYTES, dtype=torch.uint8, device="cuda").random_(0, 255)
+    c_dst = torch.empty_like(c_src)
+    for _ in range(4):
+        synth.copy_dev(c_dst, c_src)
+    torch.cuda.synchronize()
+    del c_src, c_dst
+
     # other token counts of the same config (informative)
     extra = {"gate_up_us_p50": float(np.median(gu_ms) * 1e3),
              "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
@@ -158,9 +173,9 @@ def main():
                                "scale 2.5, inter 2048); cold weights, steps rotate over "
                                f"{L} layers", "tokens_per_step": 1, "layers_rotated": L,
                    "algorithmic_bytes_per_token": TOKEN_BYTES},
-        "roofline": {"bound": "hbm", "kernel": "k_mxfp4_gate_up<1,false> (gate+up+SwiGLU, 8 routed "
-                     "+ 1 shared expert)", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "k_mxfp4_gate_up<1,false,true,true> (gate+up+SwiGLU "
+                     "+ mid quantization, 8 routed + 1 shared expert)", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": GATE_UP_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": GATE_UP_BYTES, "avg_launch_us": gu_avg_us},
         "extra": extra,
     }
@@ -179,11 +194,12 @@ def main():
         ls = lg_all[:256].cpu().numpy()
         threads = ref.max_threads()
         done, t1 = 0, time.perf_counter()
-        while done < xs.shape[0] and (time.perf_counter() - t1) < args.cpu_seconds:
-            sel, w = ref.router_topk(ls[done:done + 1], bias, base.n_used, base.route_scale,
+        while (time.perf_counter() - t1) < args.cpu_seconds:
+            i = done % xs.shape[0]
+            sel, w = ref.router_topk(ls[i:i + 1], bias, base.n_used, base.route_scale,
                                      base.route_eps, base.router_mode, base.n_group,
                                      base.topk_group)
-            ref.moe_forward(hw, xs[done:done + 1], sel, w)
+            ref.moe_forward(hw, xs[i:i + 1], sel, w)
             done += 1
         cpu_s = time.perf_counter() - t1
         result["cpu_baseline"] = {

@@ -14,6 +14,8 @@
 // q = round-half-away(x / d)).
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
+
+#include <algorithm>
 #include <math.h>
 #include <stdint.h>
 #include <string.h>
@@ -167,6 +169,15 @@ __global__ void k_q8_0(uint8_t *dst, uint64_t base, uint64_t elem0, uint64_t n_b
     if (b < n_blocks) q8_0_store(dst, base, elem0, b, cols, sigma);
 }
 
+// Plain streaming copy, 16 bytes per thread per trip: the known-traffic kernel that hardware
+// byte counters are scaled against (reads n16 * 16 bytes, writes n16 * 16 bytes).
+__global__ __launch_bounds__(256) void k_copy16(uint4 *__restrict__ dst, const uint4 *__restrict__ src,
+                                                uint64_t n16) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+        dst[i] = src[i];
+}
+
 }  // namespace
 
 extern "C" {
@@ -219,6 +230,17 @@ int dsx_synth_q8_0_dev(void *stream, uint8_t *dst, uint64_t seed, uint64_t tenso
     if (nb == 0) return 0;
     hipLaunchKernelGGL(k_q8_0, dim3((uint32_t)((nb + 127) / 128)), dim3(128), 0,
                        (hipStream_t)stream, dst, stream_base(seed, tensor_id), elem0, nb, cols, sigma);
+    return (int)hipGetLastError();
+}
+
+// dst[0 .. bytes) = src[0 .. bytes); bytes % 16 == 0, both 16-byte aligned.
+int dsx_synth_copy_dev(void *stream, void *dst, const void *src, uint64_t bytes) {
+    if (bytes == 0) return 0;
+    if (bytes % 16u || (uintptr_t)dst % 16u || (uintptr_t)src % 16u) return (int)hipErrorInvalidValue;
+    const uint64_t n16 = bytes / 16u;
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((n16 + 255) / 256, 256u * 16u);
+    hipLaunchKernelGGL(k_copy16, dim3(grid), dim3(256), 0, (hipStream_t)stream, (uint4 *)dst,
+                       (const uint4 *)src, n16);
     return (int)hipGetLastError();
 }
 

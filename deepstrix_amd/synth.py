@@ -40,6 +40,7 @@ def lib() -> C.CDLL:
         l.dsx_synth_normal_dev.argtypes = [vp, vp, u64, u64, u64, u64, f32, f32]
         l.dsx_synth_mxfp4_dev.argtypes = [vp, vp, u64, u64, u64, u64, u32, f32]
         l.dsx_synth_q8_0_dev.argtypes = [vp, vp, u64, u64, u64, u64, u32, f32]
+        l.dsx_synth_copy_dev.argtypes = [vp, vp, vp, u64]
         _lib = l
     return _lib
 
@@ -92,3 +93,13 @@ def weights_dev(fmt, seed, tensor_id, n_rows, cols, sigma=0.02, first_row=0, dev
     if rc:
         raise RuntimeError(f"dsx_synth weights: hip error {rc}")
     return out
+
+
+def copy_dev(dst, src) -> None:
+    """dst <- src with the library's plain streaming-copy kernel (byte-counter calibration)."""
+    import torch
+    assert dst.numel() * dst.element_size() == src.numel() * src.element_size()
+    rc = lib().dsx_synth_copy_dev(torch.cuda.current_stream().cuda_stream, dst.data_ptr(),
+                                  src.data_ptr(), src.numel() * src.element_size())
+    if rc:
+        raise RuntimeError(f"dsx_synth_copy_dev: hip error {rc}")
