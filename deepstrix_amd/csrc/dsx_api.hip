@@ -12,6 +12,7 @@
 
 #include "../../include/dsx_moe.h"
 #include "dsx_expert_kernels.hpp"
+#include "dsx_gemm_kernels.hpp"
 #include "dsx_misc_kernels.hpp"
 #include "dsx_q8_0_kernels.hpp"
 
@@ -60,6 +61,8 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gate_up<2, true, true, false>);
         allow_lds(k_mxfp4_gate_up<4, true, true, false>);
         allow_lds(k_mxfp4_gate_up<8, true, true, false>);
+        allow_lds(k_mxfp4_gemm<true>);
+        allow_lds(k_mxfp4_gemm<false>);
         allow_lds(k_mxfp4_down_decode<false>);
         allow_lds(k_mxfp4_down_decode<true>);
         allow_lds(k_mxfp4_down_by_expert<1, false>);
@@ -106,6 +109,34 @@ static void launch_down_be(hipStream_t st, const DownByExpertParams &p, uint32_t
     else
         hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, false>), dim3(p.n_rows / 16, max_wi),
                            dim3(kDownBeWaves * 64), lds, st, p);
+}
+
+
+// Group tables for many picks (two launches), with an optional extra group `n_expert` that
+// holds every token (slot n_used).
+int group_build_big(hipStream_t st, int32_t *group_count, int32_t *group_offset, int32_t *members,
+                    int32_t *work_items, int32_t *n_work_items, const int32_t *selected, uint32_t b,
+                    uint32_t n_used, uint32_t n_expert, uint32_t chunk, bool extra) {
+    hipLaunchKernelGGL(k_group_count, dim3(1), dim3(kGbThreads), 0, st, group_count, group_offset,
+                       work_items, n_work_items, selected, b, n_used, n_expert, chunk,
+                       extra ? 1u : 0u);
+    int rc = launched("group_count");
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_group_scatter, dim3(n_expert + (extra ? 1u : 0u)), dim3(256), 0, st, members,
+                       group_count, group_offset, selected, b, n_used, n_expert);
+    return launched("group_scatter");
+}
+
+// Grouped GEMM launch; max_wi bounds the number of work items.
+template <bool PAIR>
+int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
+    if (max_wi == 0) return DSX_OK;
+    const uint32_t per_xcd = (max_wi + 7u) / 8u;
+    const uint64_t grid = (uint64_t)8u * per_xcd * p.n_row_tiles;
+    if (grid > 0x7FFFFFFFull) return fail(DSX_ERR_INVALID_ARG, "gemm: grid too large");
+    hipLaunchKernelGGL((k_mxfp4_gemm<PAIR>), dim3((uint32_t)grid), dim3(kGemmWaves * 64), kGemmLdsBytes,
+                       st, p);
+    return launched(PAIR ? "gate_up gemm" : "down gemm");
 }
 
 }  // namespace
@@ -306,7 +337,10 @@ int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *grou
         return fail(DSX_ERR_INVALID_ARG, "moe_group_build: n_expert=%u", n_expert);
     if (b >= 65536 || n_used == 0 || n_used >= 65536)
         return fail(DSX_ERR_INVALID_ARG, "moe_group_build: b=%u n_used=%u must be below 65536", b, n_used);
-    if (chunk == 0 || chunk > 16) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..16", chunk);
+    if (chunk == 0 || chunk > 64) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..64", chunk);
+    if ((uint64_t)b * n_used > 2048u)  // many picks: histogram launch + one workgroup per expert
+        return group_build_big(S(stream), group_count, group_offset, expert_members, work_items,
+                               n_work_items, selected, b, n_used, n_expert, chunk, false);
     hipLaunchKernelGGL(k_group_build, dim3(1), dim3(kGbThreads), 0, S(stream), group_count,
                        group_offset, expert_members, work_items, n_work_items, selected, b, n_used,
                        n_expert, chunk);

@@ -392,6 +392,105 @@ __global__ __launch_bounds__(kGbThreads) void k_group_build(
 }
 
 // ---------------------------------------------------------------------------------------
+// The same tables for many picks, in two launches, plus an optional extra group with index
+// n_expert that every token belongs to (slot n_used): the dense expert riding along.
+//   k_group_count    one workgroup: histogram, prefix sums, work items
+//   k_group_scatter  one workgroup per expert: stable placement of that expert's members
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kGbThreads) void k_group_count(
+    int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
+    int32_t *__restrict__ work_items, int32_t *__restrict__ n_work_items,
+    const int32_t *__restrict__ selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
+    uint32_t chunk, uint32_t extra) {
+    __shared__ int s_count[DSX_MAX_EXPERTS_K + 1];
+    __shared__ int s_off[DSX_MAX_EXPERTS_K + 2];
+    __shared__ int s_wi_off[DSX_MAX_EXPERTS_K + 2];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t total = b * n_used;
+    const uint32_t n_groups = n_expert + (extra ? 1u : 0u);
+    for (uint32_t e = tid; e < n_groups; e += kGbThreads) s_count[e] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < total; i += kGbThreads) {
+        const int e = selected[i];
+        if (e >= 0 && (uint32_t)e < n_expert) atomicAdd(&s_count[e], 1);
+    }
+    if (extra && tid == 0) s_count[n_expert] = (int)b;
+    __syncthreads();
+    if (tid == 0) {
+        int acc = 0, wacc = 0;
+        for (uint32_t e = 0; e < n_groups; e++) {
+            s_off[e] = acc;
+            s_wi_off[e] = wacc;
+            acc += s_count[e];
+            wacc += (s_count[e] + (int)chunk - 1) / (int)chunk;
+        }
+        s_off[n_groups] = acc;
+        s_wi_off[n_groups] = wacc;
+        *n_work_items = wacc;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < n_groups; e += kGbThreads) {
+        group_count[e] = s_count[e];
+        group_offset[e] = s_off[e];
+    }
+    if (tid == 0) group_offset[n_groups] = s_off[n_groups];
+    // work items: every thread walks the groups whose items it owns
+    const uint32_t n_wi = (uint32_t)s_wi_off[n_groups];
+    for (uint32_t i = tid; i < n_wi; i += kGbThreads) {
+        // largest e with s_wi_off[e] <= i (groups without items share an offset with the next)
+        uint32_t lo = 0, hi = n_groups;
+        while (hi - lo > 1u) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if ((uint32_t)s_wi_off[mid] <= i) lo = mid; else hi = mid;
+        }
+        work_items[i] = (int)((lo << 16) | ((i - (uint32_t)s_wi_off[lo]) * chunk));
+    }
+}
+
+__global__ __launch_bounds__(256) void k_group_scatter(int32_t *__restrict__ members,
+                                                       const int32_t *__restrict__ group_count,
+                                                       const int32_t *__restrict__ group_offset,
+                                                       const int32_t *__restrict__ selected,
+                                                       uint32_t b, uint32_t n_used,
+                                                       uint32_t n_expert) {
+    __shared__ uint32_t s_cnt[4];
+    const uint32_t e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t count = (uint32_t)group_count[e];
+    if (count == 0u) return;
+    const uint32_t base = (uint32_t)group_offset[e];
+    if (e >= n_expert) {  // the extra group: every token, slot n_used
+        for (uint32_t t = tid; t < b; t += 256u) members[base + t] = (int)((t << 16) | n_used);
+        return;
+    }
+    // each wave owns a quarter of the picks (rounded to 64): count, then place
+    const uint32_t total = b * n_used;
+    const uint32_t quarter = ((total + 255u) / 256u) * 64u;
+    const uint32_t i_begin = wave * quarter, i_end = min(total, i_begin + quarter);
+    uint32_t mine = 0;
+    for (uint32_t i0 = i_begin; i0 < i_end; i0 += 64u) {
+        const uint32_t i = i0 + lane;
+        const bool hit = (i < i_end) && (selected[i] == (int)e);
+        mine += (uint32_t)__popcll(__ballot(hit));
+    }
+    if (lane == 0) s_cnt[wave] = mine;
+    __syncthreads();
+    uint32_t pos = base;
+    for (uint32_t w = 0; w < wave; w++) pos += s_cnt[w];
+    if (mine == 0u) return;
+    for (uint32_t i0 = i_begin; i0 < i_end; i0 += 64u) {
+        const uint32_t i = i0 + lane;
+        const bool hit = (i < i_end) && (selected[i] == (int)e);
+        const uint64_t mask = __ballot(hit);
+        if (hit) {
+            const uint32_t before = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+            const uint32_t t = i / n_used, slot = i - t * n_used;
+            members[pos + before] = (int)((t << 16) | slot);
+        }
+        pos += (uint32_t)__popcll(mask);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // out[t, row] = sum over slots of partials[(t * n_used + s) * n_rows + row], in slot order.
 // crates/v4flash-kernels/kernels/q2_k_accumulate_matvec_par.hip:714-730
 // `selected` (nullable): slots with a negative pick are skipped.

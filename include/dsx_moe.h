@@ -115,7 +115,7 @@ int dsx_moe_down_batched(dsx_stream_t stream, int dtype, float *out, const uint8
  * n_work_items[1].  Unlike the reference's atomic builder the order is
  * deterministic and the member table is compacted (no max_per_expert).
  * selected entries outside [0, n_expert) are skipped.  b, n_used, n_expert <
- * 65536; chunk in [1, 16]. */
+ * 65536; chunk in [1, 64] (the by-expert entry points below take chunk <= 16). */
 int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,
                         int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
                         const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
@@ -209,6 +209,11 @@ void dsx_moe_layer_destroy(dsx_moe_layer *layer);
  * launch and after the down launch, so a harness can time the dominant kernel in place. */
 int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, void *gate_up_end,
                                      void *down_end);
+/* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
+ * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
+ * gemm_min_tokens: from this many tokens on, an all-MXFP4 layer runs the grouped-GEMM path
+ * (64 token columns per work item, shared expert as an extra group). */
+int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens);
 /* Bytes of caller-provided device scratch for up to max_tokens tokens. */
 size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
 /* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],

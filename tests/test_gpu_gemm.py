@@ -1,0 +1,102 @@
+"""GPU parity of the grouped-GEMM path of the layer (many tokens per expert) against the CPU
+oracle and against the small-batch by-expert path of the same library."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from deepstrix_amd.executor import MoeLayer
+from oracle import ref
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 2e-3  # max|a-b| / max|ref|
+# The two GPU paths compute the same integer dots but sum the super-blocks in a different
+# f32 order; a mid value that lands on the other side of a rounding boundary of the second
+# quantization then moves one int8 step (1/127 of its block's largest value).
+BASE_TOL = 1e-3
+
+
+def layer_outputs(s, T, selected=None, weights=None, shift=None):
+    """(gemm path, by-expert path, oracle) outputs of one layer on the same inputs."""
+    x, logits, bias = H.host_inputs(s, T, shift)
+    dw = H.device_weights(s)
+    layer = MoeLayer(dw, T)
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    if selected is None:
+        layer.set_tuning(gemm_min_tokens=1 << 30)
+        base, sel, w = layer.run(dx, dl, want_routing=True)
+    else:
+        sel, w = torch.from_numpy(selected).cuda(), torch.from_numpy(weights).cuda()
+        layer.set_tuning(gemm_min_tokens=1 << 30)
+        base = layer.run(dx, None, selected_in=sel, weights_in=w)
+    base = base.clone()
+    layer.set_tuning(gemm_min_tokens=1)
+    got = layer.run(dx, None, selected_in=sel, weights_in=w)
+    torch.cuda.synchronize()
+    sel_h, w_h = sel.cpu().numpy(), w.cpu().numpy()
+    hw = H.host_weights(s, experts=np.unique(sel_h[sel_h >= 0]))
+    want = ref.moe_forward(hw, x, sel_h, w_h)
+    return got.cpu().numpy(), base.cpu().numpy(), want
+
+
+@pytest.mark.parametrize("T", [1, 15, 16, 17, 64, 65, 200])
+def test_small_layer_gemm_path(T):
+    s = H.Shape(1024, 512, 16, 4, router_mode=1, n_group=4, topk_group=2, route_scale=2.5,
+                bias_sigma=0.01, clamp=10.0, seed=91)
+    got, base, want = layer_outputs(s, T)
+    assert H.max_rel(got, want) < OUT_TOL
+    assert H.max_rel(got, base) < BASE_TOL
+
+
+def test_gemm_path_without_shared_expert():
+    s = H.Shape(512, 256, 8, 2, shared=False, router_mode=0, route_scale=1.5,
+                route_eps=6.103515625e-5, seed=92)
+    got, base, want = layer_outputs(s, 90)
+    assert H.max_rel(got, want) < OUT_TOL
+    assert H.max_rel(got, base) < BASE_TOL
+
+
+def test_gemm_path_all_tokens_on_the_same_experts_and_empty_slots():
+    """Worst-case imbalance: every token picks experts {0..3}; several full 64-column tiles
+    per expert plus a ragged one.  A few slots are empty (-1)."""
+    s = H.Shape(1024, 512, 16, 4, clamp=10.0, seed=93)
+    T = 150
+    sel = np.tile(np.arange(4, dtype=np.int32), (T, 1))
+    sel[5, 2] = -1
+    sel[77, 0] = -1
+    rng = np.random.default_rng(0)
+    w = rng.uniform(0.1, 1.0, (T, 4)).astype(np.float32)
+    got, base, want = layer_outputs(s, T, sel, w)
+    assert H.max_rel(got, want) < OUT_TOL
+    assert H.max_rel(got, base) < BASE_TOL
+
+
+def test_gemm_path_skewed_routing():
+    """Zipf-like logit shift: a few experts get most tokens, many get none."""
+    s = H.Shape(1024, 512, 32, 4, router_mode=1, route_scale=2.5, seed=94)
+    shift = (-1.1 * np.log(np.arange(1, 33))).astype(np.float32) * 3.0
+    got, base, want = layer_outputs(s, 300, shift=shift)
+    assert H.max_rel(got, want) < OUT_TOL
+    assert H.max_rel(got, base) < BASE_TOL
+
+
+def test_config2_v3_shape_T256_takes_the_gemm_path_by_default():
+    s = H.CFG2
+    T = 256
+    x, logits, bias = H.host_inputs(s, T)
+    dw = H.device_weights(s)
+    layer = MoeLayer(dw, T)
+    out, sel, w = layer.run(torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda(),
+                            want_routing=True)
+    torch.cuda.synchronize()
+    sel_h, w_h = sel.cpu().numpy(), w.cpu().numpy()
+    rsel, _ = H.oracle_route(s, logits, bias)
+    _, scores = ref.router_scores(logits, bias, s.router_mode, s.n_group, s.topk_group)
+    assert H.routing_mismatch_explained(sel_h, rsel, scores, s.n_used) == []
+    # the oracle on a sample of tokens (each token is independent of the others)
+    pick = np.arange(0, T, 8)
+    hw = H.host_weights(s, experts=np.unique(sel_h[pick]))
+    want = ref.moe_forward(hw, x[pick], sel_h[pick], w_h[pick])
+    assert H.max_rel(out.cpu().numpy()[pick], want) < OUT_TOL

@@ -164,7 +164,8 @@ def test_gate_up_and_down_decode_match_oracle():
 
 
 @pytest.mark.parametrize("T,E,k,chunk", [(1, 8, 3, 4), (7, 8, 3, 4), (64, 256, 8, 4), (300, 16, 4, 16),
-                                          (33, 8, 8, 1)])
+                                          (33, 8, 8, 1), (700, 16, 4, 64), (4096, 256, 8, 64),
+                                          (1000, 5, 3, 7)])
 def test_group_build_matches_oracle(T, E, k, chunk):
     rng = np.random.default_rng(T)
     sel = np.stack([rng.choice(E, k, replace=False) for _ in range(T)]).astype(np.int32)
