@@ -60,6 +60,63 @@ class Hip:
         return float(ms.value)
 
 
+FP8_MFMA_PEAK = 5.0e15   # dense FP8 MFMA, the rate class of the FP4 x FP8 instruction issued
+MXFP4_MFMA_PEAK = 10.1e15
+
+
+def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
+    """BASELINE config 3: the same layer at T = 4096 with Zipf(1.1)-skewed router logits, the
+    skew factor calibrated (on the GPU router) so that the top 10 % of experts receive about
+    half of the assignments."""
+    from deepstrix_amd import dispatch
+    from deepstrix_amd.executor import MoeLayer
+    s = H.Shape(**{**base.__dict__, "seed": base.seed + 3})
+    x, logits, _ = H.host_inputs(s, T)
+    shift = H.zipf_logit_shift(s.n_expert, 3)
+    dx = torch.from_numpy(x).cuda()
+    sel = torch.empty((T, s.n_used), dtype=torch.int32, device="cuda")
+    w = torch.empty((T, s.n_used), dtype=torch.float32, device="cuda")
+    top = max(1, round(0.1 * s.n_expert))
+
+    def share(alpha):
+        dl = torch.from_numpy((logits + alpha * shift[None, :]).astype(np.float32)).cuda()
+        dispatch.router_topk(sel, w, dl, dw.bias, s.n_expert, s.n_used, s.route_scale, s.route_eps,
+                             T, s.router_mode, s.n_group, s.topk_group)
+        cnt = np.bincount(sel.cpu().numpy().ravel(), minlength=s.n_expert)
+        return float(np.sort(cnt)[::-1][:top].sum()) / float(cnt.sum()), cnt, dl
+
+    lo, hi = 0.0, 2.0
+    for _ in range(14):
+        mid = 0.5 * (lo + hi)
+        if share(mid)[0] < 0.5:
+            lo = mid
+        else:
+            hi = mid
+    alpha = 0.5 * (lo + hi)
+    frac, cnt, dl = share(alpha)
+    layer = MoeLayer(dw, T)
+    out = torch.empty((T, s.hidden), dtype=torch.float32, device="cuda")
+    for _ in range(2):
+        layer.run(dx, dl, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        layer.run(dx, dl, out=out)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    flops = 2.0 * T * (s.n_used + 1) * 3 * s.hidden * s.inter
+    del layer
+    return {"tokens_per_s": T / dt, "ms_per_layer": dt * 1e3, "zipf_alpha": alpha,
+            "top10pct_share": frac, "max_group": int(cnt.max()), "empty_experts": int((cnt == 0).sum()),
+            "column_tiles_of_64": int(np.ceil(cnt / 64).sum()) + T // 64,
+            "useful_flop": flops, "useful_TFLOPs": flops / dt / 1e12,
+            "mfma_issued": "v_mfma_scale_f32_16x16x128_f8f6f4, A = FP4 weights, B = FP8 planes of the "
+                           "int8 activations (two instructions per product)",
+            "mfma_frac_useful_vs_fp8_peak": flops / dt / FP8_MFMA_PEAK,
+            "mfma_frac_issued_vs_fp8_peak": 2.0 * flops / dt / FP8_MFMA_PEAK,
+            "mfma_frac_useful_vs_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,6 +124,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--layers", type=int, default=4, help="independent layers the steps rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the T=4096 prefill leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -156,6 +214,9 @@ def main():
             layers[r % L].run(xs, ls, out=o)
         torch.cuda.synchronize()
         extra[f"us_per_token_T{T}"] = (time.perf_counter() - t1) * 1e6 / reps / T
+
+    if not args.no_prefill:
+        extra["prefill_T4096"] = prefill_leg(layers[0].w, base, H, torch, np)
 
     result = {
         "metric": "moe_layer_us_per_token_T1",

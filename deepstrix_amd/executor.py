@@ -84,8 +84,11 @@ class MoeLayer:
     def __del__(self):
         h = getattr(self, "_h", None)
         if h:
-            lib().dsx_moe_layer_destroy(h)
             self._h = None
+            try:
+                lib().dsx_moe_layer_destroy(h)
+            except Exception:  # interpreter shutdown: the module globals are already gone
+                pass
 
     def set_profile_events(self, gate_up_begin=None, gate_up_end=None, down_end=None):
         """hipEvent_t handles (ints) recorded around the gate/up launch and after down."""

@@ -137,3 +137,13 @@ def routing_mismatch_explained(sel_gpu, sel_ref, scores, n_used, tol=1e-4):
         if gap > tol:
             bad.append((t, float(gap)))
     return bad
+
+
+def zipf_logit_shift(n_expert: int, seed: int, s: float = 1.1) -> np.ndarray:
+    """-s * ln(rank) under a seeded permutation of the experts (BASELINE config 3: added to
+    N(0,1) logits with a factor chosen so that the top 10 % of experts get ~50 % of the picks)."""
+    rng = np.random.default_rng(seed)
+    perm = rng.permutation(n_expert)
+    shift = np.empty(n_expert, np.float32)
+    shift[perm] = (-s * np.log(np.arange(1, n_expert + 1))).astype(np.float32)
+    return shift
