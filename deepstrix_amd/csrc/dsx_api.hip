@@ -141,8 +141,8 @@ int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
 
 }  // namespace
 
-int dsx::q8_0_unsupported(const char *what) {
-    return fail(DSX_ERR_UNSUPPORTED, "%s: Q8_0 expert kernels are not built", what);
+int dsx::q8_0_fail(int code, const char *what, const char *why) {
+    return fail(code, "%s: %s", what, why);
 }
 
 extern "C" {

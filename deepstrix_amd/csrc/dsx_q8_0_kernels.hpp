@@ -1,39 +1,375 @@
-// dsx_q8_0_kernels.hpp -- Q8_0 expert products (int8 MFMA).  Filled in below.
+// dsx_q8_0_kernels.hpp -- Q8_0 expert products on gfx950.
+//
+// Weights: engine rows [blocks x f16 d][blocks x 32 i8] (crates/v4flash-kernels/src/weights.rs:
+// 225-240).  Activations: rows [k i8][k/32 f32 scales] made by k_q8_0_quantize_rows
+// (crates/v4flash-kernels/kernels/q8_0_matvec.hip:150-177).  The product of one block is
+// exact in int32 (v_dot4_i32_i8), scaled by f16(d_w) * xscale in f32
+// (crates/v4flash-kernels/kernels/q8_0_matvec.hip:64-104).
+//
+// A wave reads one weight row front to back: lane l takes blocks l, l + 64, ... (32 int8 =
+// 32 contiguous bytes per lane, 2 KiB contiguous per wave load step), multiplies them with
+// the matching activation blocks of every token column (LDS), and the 64 partial sums of a
+// (row, column) are added by a butterfly.  A workgroup of four waves owns 16 rows, four per
+// wave.  These are streaming kernels for few columns (decode and small batches).
 #pragma once
 
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include "../../include/dsx_moe.h"
+#include "dsx_device.hpp"
+#include "dsx_quant.hpp"
 
 namespace dsx {
 
-int q8_0_unsupported(const char *what);
+int q8_0_fail(int code, const char *what, const char *why);
 
-inline void q8_0_raise_lds_limits() {}
+constexpr int kQ8Waves = 4;
+constexpr int kQ8RowsPerWg = 16;
+constexpr size_t kQ8LdsBudget = 140 * 1024;
 
-inline int q8_0_gate_up_decode(hipStream_t, float *, const uint8_t *, const uint8_t *,
-                               const uint8_t *, const float *, const int32_t *, const uint8_t *,
-                               const uint8_t *, float, uint64_t, uint64_t, uint32_t, float,
-                               uint32_t, uint32_t) {
-    return q8_0_unsupported("moe_gate_up_batch");
+__host__ __device__ inline uint32_t q8_0_act_row_bytes(uint32_t n_blocks) { return n_blocks * 36u; }
+
+struct Q8Params {
+    float *dst;                       // mid / partials [dest rows, n_rows], or out [n_rows]
+    const uint8_t *w0, *w1;           // [n_expert] experts: gate and up, or down in w0
+    const uint8_t *sh_w0, *sh_w1;     // decode: the extra slot n_used (weight 1), or null
+    uint64_t bpe0, bpe1;
+    const uint8_t *xq;                // activation rows, x_stride bytes apart
+    const float *ew;
+    const int32_t *selected;          // decode
+    const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
+    uint32_t x_stride, n_used, chunk, n_rows, n_blocks;
+    float clamp, sh_clamp;
+};
+
+// The lane's share of `row . x[c]` for NT columns, over all of its blocks.
+template <int NT>
+__device__ __forceinline__ void q8_0_row_partial(float (&acc)[NT], const uint8_t *__restrict__ row,
+                                                 const uint8_t *lds_x, uint32_t col_stride,
+                                                 uint32_t n_blocks, uint32_t lane) {
+    const uint8_t *quants = row + (size_t)n_blocks * 2u;
+    for (uint32_t b0 = 0; b0 < n_blocks; b0 += 64u) {
+        const uint32_t b = b0 + lane;
+        const bool live = b < n_blocks;
+        const uint32_t bb = live ? b : n_blocks - 1u;  // clamped: the load stays in the row
+        const U2A4 w0 = gload8(quants + (size_t)bb * 32u);
+        const U2A4 w1 = gload8(quants + (size_t)bb * 32u + 8u);
+        const U2A4 w2 = gload8(quants + (size_t)bb * 32u + 16u);
+        const U2A4 w3 = gload8(quants + (size_t)bb * 32u + 24u);
+        const uint16_t dbits = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(row + (size_t)bb * 2u);
+        const float dw = live ? __half2float(__ushort_as_half(dbits)) : 0.0f;
+#pragma unroll
+        for (int c = 0; c < NT; c++) {
+            const uint8_t *xc = lds_x + (size_t)c * col_stride;
+            const uint4 x0 = *(const uint4 *)(xc + bb * 32u);
+            const uint4 x1 = *(const uint4 *)(xc + bb * 32u + 16u);
+            const float xs = *(const float *)(xc + n_blocks * 32u + bb * 4u);
+            int s = 0;
+            s = __builtin_amdgcn_sdot4((int)w0.x, (int)x0.x, s, false);
+            s = __builtin_amdgcn_sdot4((int)w0.y, (int)x0.y, s, false);
+            s = __builtin_amdgcn_sdot4((int)w1.x, (int)x0.z, s, false);
+            s = __builtin_amdgcn_sdot4((int)w1.y, (int)x0.w, s, false);
+            s = __builtin_amdgcn_sdot4((int)w2.x, (int)x1.x, s, false);
+            s = __builtin_amdgcn_sdot4((int)w2.y, (int)x1.y, s, false);
+            s = __builtin_amdgcn_sdot4((int)w3.x, (int)x1.z, s, false);
+            s = __builtin_amdgcn_sdot4((int)w3.y, (int)x1.w, s, false);
+            acc[c] += dw * xs * (float)s;
+        }
+    }
 }
-inline int q8_0_down_decode(hipStream_t, float *, const uint8_t *, const uint8_t *, const int32_t *,
-                            const uint8_t *, uint64_t, uint32_t, uint32_t, uint32_t, uint32_t) {
-    return q8_0_unsupported("moe_down_batched");
+
+// Copies `n_cols` activation rows (row j from src(j)) into LDS, col_stride bytes apart.
+template <typename Src>
+__device__ __forceinline__ void q8_0_stage(uint8_t *lds_x, uint32_t n_cols, uint32_t row_bytes,
+                                           uint32_t tid, const Src src) {
+    const uint32_t per = row_bytes / 16u;
+    for (uint32_t q = tid; q < n_cols * per; q += kQ8Waves * 64u) {
+        const uint32_t j = q / per, c = q - j * per;
+        *(uint4 *)(lds_x + (size_t)j * row_bytes + (size_t)c * 16u) =
+            *(const uint4 *)(src(j) + (size_t)c * 16u);
+    }
 }
-inline int q8_0_gate_up_by_expert(hipStream_t, float *, const uint8_t *, const uint8_t *,
-                                  const uint8_t *, const float *, const int32_t *, const int32_t *,
-                                  const int32_t *, const int32_t *, const int32_t *, uint32_t,
-                                  uint64_t, uint64_t, uint32_t, uint32_t, float, uint32_t,
-                                  uint32_t) {
-    return q8_0_unsupported("moe_gate_up_chunked_rows");
+
+// ---------------------------------------------------------------------------------------
+// gate/up + SwiGLU.  BY_EXPERT = false: one token, grid.y = slot (slot n_used = the extra
+// expert).  BY_EXPERT = true: grid.y = work item, columns = its members.
+// crates/v4flash-kernels/src/het/dispatch.rs:26-66, 534-570 (Q8_0 arms)
+// ---------------------------------------------------------------------------------------
+template <int NT, bool BY_EXPERT>
+__global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_gate_up(const Q8Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];
+    __shared__ uint32_t s_tok[NT];
+    __shared__ uint32_t s_dest[NT];
+    __shared__ float s_ew[NT];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y;
+    const uint32_t row_bytes = q8_0_act_row_bytes(p.n_blocks);
+    const uint8_t *g_e, *u_e;
+    uint32_t cnt = 1;
+    float clamp = p.clamp;
+    if (BY_EXPERT) {
+        if ((int)item >= *p.n_work_items) return;
+        const uint32_t wi = (uint32_t)p.work_items[item];
+        const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
+        cnt = min(min(p.chunk, (uint32_t)NT), (uint32_t)p.group_count[e] - start);
+        const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+        if (tid < cnt) {
+            const uint32_t m = (uint32_t)p.members[mbase + tid];
+            const uint32_t t = m >> 16, slot = m & 0xFFFFu;
+            s_tok[tid] = t;
+            s_dest[tid] = t * p.n_used + slot;
+            s_ew[tid] = p.ew[t * p.n_used + slot];
+        }
+        g_e = p.w0 + (uint64_t)e * p.bpe0;
+        u_e = p.w1 + (uint64_t)e * p.bpe1;
+    } else {
+        if (item < p.n_used) {
+            const int e = p.selected[item];
+            if (e < 0) {  // empty slot: defined output
+                if (tid < (uint32_t)kQ8RowsPerWg) p.dst[(uint64_t)item * p.n_rows + row0 + tid] = 0.0f;
+                return;
+            }
+            g_e = p.w0 + (uint64_t)e * p.bpe0;
+            u_e = p.w1 + (uint64_t)e * p.bpe1;
+            if (tid == 0) s_ew[0] = p.ew[item];
+        } else {
+            g_e = p.sh_w0;
+            u_e = p.sh_w1;
+            clamp = p.sh_clamp;
+            if (tid == 0) s_ew[0] = 1.0f;
+        }
+        if (tid == 0) {
+            s_tok[0] = 0;
+            s_dest[0] = item;
+        }
+    }
+    __syncthreads();
+    q8_0_stage(lds_x, cnt, row_bytes, tid,
+               [&](uint32_t j) { return p.xq + (uint64_t)s_tok[j] * p.x_stride; });
+    __syncthreads();
+
+    const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
+    for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
+        const uint32_t row = row0 + r;
+        float g[NT], u[NT];
+#pragma unroll
+        for (int c = 0; c < NT; c++) g[c] = u[c] = 0.0f;
+        q8_0_row_partial<NT>(g, g_e + (uint64_t)row * wstride, lds_x, row_bytes, p.n_blocks, lane);
+        q8_0_row_partial<NT>(u, u_e + (uint64_t)row * wstride, lds_x, row_bytes, p.n_blocks, lane);
+#pragma unroll
+        for (int c = 0; c < NT; c++) {
+            const float gs = wave_sum_f32(g[c]), us = wave_sum_f32(u[c]);
+            if (lane == 0 && (uint32_t)c < cnt)
+                p.dst[(uint64_t)s_dest[c] * p.n_rows + row] = swiglu_clamp(gs, us, clamp, s_ew[c]);
+        }
+    }
 }
-inline int q8_0_down_by_expert(hipStream_t, float *, const uint8_t *, const uint8_t *,
-                               const int32_t *, const int32_t *, const int32_t *, const int32_t *,
-                               const int32_t *, uint32_t, uint64_t, uint32_t, uint32_t, uint32_t,
-                               uint32_t, uint32_t) {
-    return q8_0_unsupported("moe_down_by_expert");
+
+// ---------------------------------------------------------------------------------------
+// down, one token: out[row] = sum over slots (slot order) of down_e(slot)[row] . midq[slot].
+// crates/v4flash-kernels/src/het/dispatch.rs:121-150 (Q8_0 arm)
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_decode(const Q8Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];
+    __shared__ int s_sel[DSX_MAX_USED + 1];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg;
+    const uint32_t row_bytes = q8_0_act_row_bytes(p.n_blocks);
+    const uint32_t n_slots = p.n_used + (p.sh_w0 ? 1u : 0u);
+    if (tid < p.n_used) s_sel[tid] = p.selected[tid];
+    q8_0_stage(lds_x, n_slots, row_bytes, tid,
+               [&](uint32_t j) { return p.xq + (uint64_t)j * p.x_stride; });
+    __syncthreads();
+    const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
+    for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
+        const uint32_t row = row0 + r;
+        float total = 0.0f;
+        for (uint32_t s = 0; s < n_slots; s++) {
+            const uint8_t *w;
+            if (s < p.n_used) {
+                const int e = s_sel[s];
+                if (e < 0) continue;
+                w = p.w0 + (uint64_t)e * p.bpe0;
+            } else {
+                w = p.sh_w0;
+            }
+            float a[1] = {0.0f};
+            q8_0_row_partial<1>(a, w + (uint64_t)row * wstride, lds_x + (size_t)s * row_bytes, row_bytes,
+                                p.n_blocks, lane);
+            total += wave_sum_f32(a[0]);
+        }
+        if (lane == 0) p.dst[row] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// down, by expert: partials[(t * n_used + slot) * n_rows + row] = down_e[row] . midq[t, slot]
+// crates/v4flash-kernels/src/het/dispatch.rs:580-620 (Q8_0 arm)
+// ---------------------------------------------------------------------------------------
+template <int NT>
+__global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_by_expert(const Q8Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];
+    __shared__ uint32_t s_dest[NT];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y;
+    const uint32_t row_bytes = q8_0_act_row_bytes(p.n_blocks);
+    if ((int)item >= *p.n_work_items) return;
+    const uint32_t wi = (uint32_t)p.work_items[item];
+    const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
+    const uint32_t cnt = min(min(p.chunk, (uint32_t)NT), (uint32_t)p.group_count[e] - start);
+    const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+    if (tid < cnt) {
+        const uint32_t m = (uint32_t)p.members[mbase + tid];
+        s_dest[tid] = (m >> 16) * p.n_used + (m & 0xFFFFu);
+    }
+    __syncthreads();
+    q8_0_stage(lds_x, cnt, row_bytes, tid,
+               [&](uint32_t j) { return p.xq + (uint64_t)s_dest[j] * p.x_stride; });
+    __syncthreads();
+    const uint8_t *w_e = p.w0 + (uint64_t)e * p.bpe0;
+    const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
+    for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
+        const uint32_t row = row0 + r;
+        float a[NT];
+#pragma unroll
+        for (int c = 0; c < NT; c++) a[c] = 0.0f;
+        q8_0_row_partial<NT>(a, w_e + (uint64_t)row * wstride, lds_x, row_bytes, p.n_blocks, lane);
+#pragma unroll
+        for (int c = 0; c < NT; c++) {
+            const float v = wave_sum_f32(a[c]);
+            if (lane == 0 && (uint32_t)c < cnt) p.dst[(uint64_t)s_dest[c] * p.n_rows + row] = v;
+        }
+    }
+}
+
+// ---- host side ----------------------------------------------------------------------------
+inline void q8_0_raise_lds_limits() {
+    const int lim = 160 * 1024 - 16 * 1024;
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gate_up<1, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gate_up<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gate_up<2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gate_up<4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gate_up<8, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_down_decode, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_down_by_expert<1>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_down_by_expert<2>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_down_by_expert<4>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_down_by_expert<8>, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+}
+
+inline int q8_0_check(const char *what, uint32_t n_rows, uint32_t n_blocks, const void *w0,
+                      const void *w1, uint64_t bpe0, uint64_t bpe1, const void *xq, uint32_t x_stride,
+                      uint32_t n_cols) {
+    if (n_rows == 0 || n_rows % kQ8RowsPerWg != 0)
+        return q8_0_fail(DSX_ERR_SHAPE, what, "n_rows must be a multiple of 16");
+    if (n_blocks == 0 || n_blocks % 4 != 0)
+        return q8_0_fail(DSX_ERR_SHAPE, what, "Q8_0 rows need k % 128 == 0");
+    if ((uintptr_t)w0 % 8 || (uintptr_t)w1 % 8 || bpe0 % 8 || bpe1 % 8)
+        return q8_0_fail(DSX_ERR_SHAPE, what, "Q8_0 weights must be 8-byte aligned");
+    if ((uintptr_t)xq % 16 || x_stride % 16 || x_stride < q8_0_act_row_bytes(n_blocks))
+        return q8_0_fail(DSX_ERR_SHAPE, what, "Q8_0 activation rows must be 16-byte aligned, stride >= 36 * blocks");
+    if ((size_t)n_cols * q8_0_act_row_bytes(n_blocks) > kQ8LdsBudget)
+        return q8_0_fail(DSX_ERR_UNSUPPORTED, what, "activation columns exceed LDS staging");
+    return DSX_OK;
+}
+
+inline int q8_0_pick_nt(uint32_t chunk) { return chunk <= 1 ? 1 : chunk <= 2 ? 2 : chunk <= 4 ? 4 : 8; }
+
+inline int q8_0_gate_up_decode(hipStream_t st, float *mid, const uint8_t *gate, const uint8_t *up,
+                               const uint8_t *xq, const float *ew, const int32_t *selected,
+                               const uint8_t *sh_gate, const uint8_t *sh_up, float sh_clamp,
+                               uint64_t gbpe, uint64_t ubpe, uint32_t n_used, float clamp,
+                               uint32_t n_rows, uint32_t n_blocks) {
+    int rc = q8_0_check("moe_gate_up_batch", n_rows, n_blocks, gate, up, gbpe, ubpe, xq,
+                        q8_0_act_row_bytes(n_blocks), 1);
+    if (rc) return rc;
+    Q8Params p{};
+    p.dst = mid; p.w0 = gate; p.w1 = up; p.sh_w0 = sh_gate; p.sh_w1 = sh_up; p.bpe0 = gbpe; p.bpe1 = ubpe;
+    p.xq = xq; p.ew = ew; p.selected = selected; p.x_stride = q8_0_act_row_bytes(n_blocks);
+    p.n_used = n_used; p.chunk = 1; p.n_rows = n_rows; p.n_blocks = n_blocks; p.clamp = clamp;
+    p.sh_clamp = sh_clamp;
+    const uint32_t n_slots = n_used + (sh_gate ? 1u : 0u);
+    hipLaunchKernelGGL((k_q8_0_gate_up<1, false>), dim3(n_rows / kQ8RowsPerWg, n_slots),
+                       dim3(kQ8Waves * 64), q8_0_act_row_bytes(n_blocks), st, p);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DSX_OK : q8_0_fail((int)e, "moe_gate_up_batch", hipGetErrorString(e));
+}
+
+inline int q8_0_down_decode(hipStream_t st, float *out, const uint8_t *down, const uint8_t *xq,
+                            const int32_t *selected, const uint8_t *sh_down, uint64_t dbpe,
+                            uint32_t xq_slot_stride, uint32_t n_used, uint32_t n_rows,
+                            uint32_t n_blocks_in) {
+    const uint32_t n_slots = n_used + (sh_down ? 1u : 0u);
+    int rc = q8_0_check("moe_down_batched", n_rows, n_blocks_in, down, sh_down, dbpe, 0, xq,
+                        xq_slot_stride, n_slots);
+    if (rc) return rc;
+    Q8Params p{};
+    p.dst = out; p.w0 = down; p.sh_w0 = sh_down; p.bpe0 = dbpe; p.xq = xq; p.selected = selected;
+    p.x_stride = xq_slot_stride; p.n_used = n_used; p.n_rows = n_rows; p.n_blocks = n_blocks_in;
+    hipLaunchKernelGGL(k_q8_0_down_decode, dim3(n_rows / kQ8RowsPerWg), dim3(kQ8Waves * 64),
+                       (size_t)n_slots * q8_0_act_row_bytes(n_blocks_in), st, p);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DSX_OK : q8_0_fail((int)e, "moe_down_batched", hipGetErrorString(e));
+}
+
+inline int q8_0_gate_up_by_expert(hipStream_t st, float *mid, const uint8_t *gate, const uint8_t *up,
+                                  const uint8_t *xq, const float *ew, const int32_t *group_count,
+                                  const int32_t *group_offset, const int32_t *members,
+                                  const int32_t *work_items, const int32_t *n_work_items,
+                                  uint32_t max_wi, uint64_t gbpe, uint64_t ubpe, uint32_t n_used,
+                                  uint32_t chunk, float clamp, uint32_t n_rows, uint32_t n_blocks) {
+    if (chunk > 8) return q8_0_fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows", "Q8_0 takes chunk <= 8");
+    const int nt = q8_0_pick_nt(chunk);
+    int rc = q8_0_check("moe_gate_up_chunked_rows", n_rows, n_blocks, gate, up, gbpe, ubpe, xq,
+                        q8_0_act_row_bytes(n_blocks), (uint32_t)nt);
+    if (rc) return rc;
+    Q8Params p{};
+    p.dst = mid; p.w0 = gate; p.w1 = up; p.bpe0 = gbpe; p.bpe1 = ubpe; p.xq = xq; p.ew = ew;
+    p.group_count = group_count; p.group_offset = group_offset; p.members = members;
+    p.work_items = work_items; p.n_work_items = n_work_items;
+    p.x_stride = q8_0_act_row_bytes(n_blocks); p.n_used = n_used; p.chunk = chunk; p.n_rows = n_rows;
+    p.n_blocks = n_blocks; p.clamp = clamp;
+    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi), block(kQ8Waves * 64);
+    const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks);
+    switch (nt) {
+        case 1: hipLaunchKernelGGL((k_q8_0_gate_up<1, true>), grid, block, lds, st, p); break;
+        case 2: hipLaunchKernelGGL((k_q8_0_gate_up<2, true>), grid, block, lds, st, p); break;
+        case 4: hipLaunchKernelGGL((k_q8_0_gate_up<4, true>), grid, block, lds, st, p); break;
+        default: hipLaunchKernelGGL((k_q8_0_gate_up<8, true>), grid, block, lds, st, p); break;
+    }
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DSX_OK : q8_0_fail((int)e, "moe_gate_up_chunked_rows", hipGetErrorString(e));
+}
+
+inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *down, const uint8_t *xq,
+                               const int32_t *group_count, const int32_t *group_offset,
+                               const int32_t *members, const int32_t *work_items,
+                               const int32_t *n_work_items, uint32_t max_wi, uint64_t dbpe,
+                               uint32_t xq_slot_stride, uint32_t n_used, uint32_t chunk,
+                               uint32_t n_rows, uint32_t n_blocks_in) {
+    if (chunk > 8) return q8_0_fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert", "Q8_0 takes chunk <= 8");
+    const int nt = q8_0_pick_nt(chunk);
+    int rc = q8_0_check("moe_down_by_expert", n_rows, n_blocks_in, down, nullptr, dbpe, 0, xq,
+                        xq_slot_stride, (uint32_t)nt);
+    if (rc) return rc;
+    Q8Params p{};
+    p.dst = partials; p.w0 = down; p.bpe0 = dbpe; p.xq = xq;
+    p.group_count = group_count; p.group_offset = group_offset; p.members = members;
+    p.work_items = work_items; p.n_work_items = n_work_items;
+    p.x_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk; p.n_rows = n_rows;
+    p.n_blocks = n_blocks_in;
+    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi), block(kQ8Waves * 64);
+    const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks_in);
+    switch (nt) {
+        case 1: hipLaunchKernelGGL(k_q8_0_down_by_expert<1>, grid, block, lds, st, p); break;
+        case 2: hipLaunchKernelGGL(k_q8_0_down_by_expert<2>, grid, block, lds, st, p); break;
+        case 4: hipLaunchKernelGGL(k_q8_0_down_by_expert<4>, grid, block, lds, st, p); break;
+        default: hipLaunchKernelGGL(k_q8_0_down_by_expert<8>, grid, block, lds, st, p); break;
+    }
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DSX_OK : q8_0_fail((int)e, "moe_down_by_expert", hipGetErrorString(e));
 }
 
 }  // namespace dsx
