@@ -232,7 +232,7 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
                                const uint8_t *sh_up, float sh_clamp, uint64_t gbpe, uint64_t ubpe,
                                uint32_t n_used, float clamp, uint32_t n_rows, uint32_t n_blocks,
                                bool staged = false, uint8_t *midp = nullptr,
-                               int32_t *counters = nullptr) {
+                               int32_t *counters = nullptr, uint32_t n_tokens = 1) {
     if (n_used == 0 && !sh_gate) return DSX_OK;
     if (!mid || !gate || !up || !xq || !ew || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: null pointer");
@@ -263,11 +263,11 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
         p.midp = midp;
         p.counters = counters;
         p.midp_row_bytes = staged_row_bytes(n_rows / 256);
-        hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, true, true>), dim3(n_rows / 16, n_slots),
-                           dim3(kGuWaves * 64), lds, st, p);
+        hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, true, true>),
+                           dim3(n_rows / 16, n_slots * n_tokens), dim3(kGuWaves * 64), lds, st, p);
     } else {
-        hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, false, false>), dim3(n_rows / 16, n_slots),
-                           dim3(kGuWaves * 64), lds, st, p);
+        hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, false, false>),
+                           dim3(n_rows / 16, n_slots * n_tokens), dim3(kGuWaves * 64), lds, st, p);
     }
     return launched("moe_gate_up_batch");
 }
@@ -283,7 +283,8 @@ int dsx_moe_gate_up_batch(dsx_stream_t stream, int dtype, float *mid, const uint
 static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t *down,
                             const uint8_t *xq, const int32_t *selected, const uint8_t *sh_down,
                             uint64_t dbpe, uint32_t xq_slot_stride, uint32_t n_used,
-                            uint32_t n_rows, uint32_t n_blocks_in, bool staged = false) {
+                            uint32_t n_rows, uint32_t n_blocks_in, bool staged = false,
+                            uint32_t n_tokens = 1) {
     if (!out || !down || !xq || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: null pointer");
     if (n_used > DSX_MAX_USED) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_used=%u", n_used);
@@ -311,9 +312,9 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.n_slots = n_slots;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
     if (staged)
-        hipLaunchKernelGGL(k_mxfp4_down_decode<true>, dim3(n_rows / 16), dim3(kDownWaves * 64), lds, st, p);
+        hipLaunchKernelGGL(k_mxfp4_down_decode<true>, dim3(n_rows / 16, n_tokens), dim3(kDownWaves * 64), lds, st, p);
     else
-        hipLaunchKernelGGL(k_mxfp4_down_decode<false>, dim3(n_rows / 16), dim3(kDownWaves * 64), lds, st, p);
+        hipLaunchKernelGGL(k_mxfp4_down_decode<false>, dim3(n_rows / 16, n_tokens), dim3(kDownWaves * 64), lds, st, p);
     return launched("moe_down_batched");
 }
 

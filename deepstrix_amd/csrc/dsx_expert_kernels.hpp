@@ -150,9 +150,12 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         gate_e = p.gate + (uint64_t)e * p.gbpe;
         up_e = p.up + (uint64_t)e * p.ubpe;
     } else {
+        // decode: item = token * n_slots + slot; slot n_used is the extra (shared) expert
         cnt = 1;
-        if (item < p.n_used) {
-            const int e = p.selected[item];
+        const uint32_t n_slots = p.n_used + (p.sh_gate ? 1u : 0u);
+        const uint32_t t = item / n_slots, slot = item - t * n_slots;
+        if (slot < p.n_used) {
+            const int e = p.selected[t * p.n_used + slot];
             if (e < 0) {  // empty slot: defined output, nothing to compute
                 if (tid < 16) p.mid[(uint64_t)item * p.n_rows + row0 + tid] = 0.0f;
                 if (FUSE_MIDQ && row0 % 256u == 0u && wave == 0) {
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
             }
             gate_e = p.gate + (uint64_t)e * p.gbpe;
             up_e = p.up + (uint64_t)e * p.ubpe;
-            if (tid == 0) s_ew[0] = p.ew[item];
+            if (tid == 0) s_ew[0] = p.ew[t * p.n_used + slot];
         } else {
             gate_e = p.sh_gate;
             up_e = p.sh_up;
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
             if (tid == 0) s_ew[0] = 1.0f;
         }
         if (tid == 0) {
-            s_tok[0] = 0;
+            s_tok[0] = t;
             s_dest[0] = (int)item;
         }
     }
@@ -196,17 +199,18 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     }
 
     // ---- activations into LDS -----------------------------------------------------------
-    if (BY_EXPERT) __syncthreads();  // s_tok visible
+    __syncthreads();  // s_tok visible
     if (STAGED) {
         if (BY_EXPERT)
             stage_copy<NT, kGuWaves * 64>(tiles, s_yd, cnt, p.n_blocks, tid,
                                           StageMembers{p.xq, p.xq_row_bytes, s_tok});
         else
-            stage_copy<NT, kGuWaves * 64>(tiles, s_yd, 1u, p.n_blocks, tid, StageDecode{p.xq});
+            stage_copy<NT, kGuWaves * 64>(tiles, s_yd, 1u, p.n_blocks, tid,
+                                          StageDecode{p.xq + (uint64_t)s_tok[0] * p.xq_row_bytes});
     } else {
         for (uint32_t pr = wave; pr < cnt * p.n_blocks; pr += kGuWaves) {
             const uint32_t j = pr / p.n_blocks, b = pr - j * p.n_blocks;
-            const uint32_t tok = BY_EXPERT ? s_tok[j] : 0u;
+            const uint32_t tok = s_tok[j];
             const uint8_t *blk = p.xq + (uint64_t)tok * p.xq_row_bytes + (uint64_t)b * kQ8kBytes;
             stage_q8k_block<NT>(tiles + (size_t)b * 512u * NT, s_yd + b * NT + j, blk, j, lane);
         }
@@ -305,10 +309,10 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
 constexpr int kDownWaves = 8;
 
 struct DownDecodeParams {
-    float *out;             // [n_rows]
+    float *out;             // [n_tokens, n_rows]; grid.y = token
     const uint8_t *down;    // [n_expert] experts, stride dbpe
     const uint8_t *xq;      // slot-major activation rows (Q8_K or staged), xq_slot_stride apart
-    const int32_t *selected;  // [n_used]
+    const int32_t *selected;  // [n_tokens, n_used]
     const uint8_t *sh_down;   // extra slot n_used, or null
     uint64_t dbpe;
     uint32_t xq_slot_stride, n_used, n_slots, n_rows, n_blocks_in;
@@ -330,10 +334,14 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     const uint32_t row0 = blockIdx.x * 16u;
     const uint32_t r = lane & 15u, kb = lane >> 4;
     const uint64_t row_off = (uint64_t)(row0 + r) * nb * kSuperBytes;
+    // blockIdx.y = token: its picks, its n_slots activation rows, its output row
+    const int32_t *selected = p.selected + (uint64_t)blockIdx.y * p.n_used;
+    const uint8_t *xq = p.xq + (uint64_t)blockIdx.y * p.n_slots * p.xq_slot_stride;
+    float *out = p.out + (uint64_t)blockIdx.y * p.n_rows;
 
     auto unit_ptr = [&](uint32_t un) -> const uint8_t * {
         const uint32_t slot = un / nb, b = un - slot * nb;
-        const int e = (slot < p.n_used) ? p.selected[slot] : 0;
+        const int e = (slot < p.n_used) ? selected[slot] : 0;
         const uint8_t *base = (slot < p.n_used) ? p.down + (uint64_t)(e < 0 ? 0 : e) * p.dbpe
                                                 : p.sh_down;
         return base + row_off + (uint64_t)b * kSuperBytes;
@@ -348,14 +356,14 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     if (un + 3 * kDownWaves < units) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
     if (un + 4 * kDownWaves < units) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
 
-    if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? p.selected[tid] : 0;
+    if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? selected[tid] : 0;
     if (STAGED) {
         stage_copy<1, kDownWaves * 64>(tiles, s_yd, p.n_slots, nb, tid,
-                                       StageSlots{p.xq, p.xq_slot_stride, nb});
+                                       StageSlots{xq, p.xq_slot_stride, nb});
     } else {
         for (uint32_t pr = wave; pr < units; pr += kDownWaves) {
             const uint32_t slot = pr / nb, b = pr - slot * nb;
-            const uint8_t *blk = p.xq + (uint64_t)slot * p.xq_slot_stride + (uint64_t)b * kQ8kBytes;
+            const uint8_t *blk = xq + (uint64_t)slot * p.xq_slot_stride + (uint64_t)b * kQ8kBytes;
             stage_q8k_block<1>(tiles + (size_t)pr * 512u, s_yd + pr, blk, 0, lane);
         }
     }
@@ -392,7 +400,7 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
         float s = 0.0f;
 #pragma unroll
         for (int wv = 0; wv < kDownWaves; wv++) s += s_red[wv][i][l];
-        p.out[row0 + tid] = s;
+        out[row0 + tid] = s;
     }
 }
 

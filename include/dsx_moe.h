@@ -212,8 +212,11 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
 /* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
  * gemm_min_tokens: from this many tokens on, an all-MXFP4 layer runs the grouped-GEMM path
- * (64 token columns per work item, shared expert as an extra group). */
-int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens);
+ * (64 token columns per work item, shared expert as an extra group).
+ * decode_max_tokens: up to this many tokens, an all-MXFP4 layer runs the one-token decode
+ * kernels once per token inside the same launches (no grouping by expert). */
+int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
+                             uint32_t decode_max_tokens);
 /* Bytes of caller-provided device scratch for up to max_tokens tokens. */
 size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
 /* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],

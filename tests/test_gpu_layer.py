@@ -57,6 +57,7 @@ def test_pinned_routing_and_row_independence():
     x, logits, bias = H.host_inputs(s, T)
     dw = H.device_weights(s)
     layer = MoeLayer(dw, T)
+    layer.set_tuning(decode_max_tokens=1)   # keep the two-token call on the by-expert path too
     dx = torch.from_numpy(x).cuda()
     out, sel, w = layer.run(dx, torch.from_numpy(logits).cuda(), want_routing=True)
     out2 = layer.run(dx, None, selected_in=sel, weights_in=w)
@@ -64,6 +65,36 @@ def test_pinned_routing_and_row_independence():
     pair = layer.run(dx[2:4].contiguous(), None, selected_in=sel[2:4].contiguous(),
                      weights_in=w[2:4].contiguous())
     assert torch.equal(pair, out[2:4])
+
+
+@pytest.mark.parametrize("T", [2, 3, 4, 7])
+def test_per_token_decode_path_equals_by_expert_path(T):
+    """Up to decode_max_tokens tokens run the decode kernels once per token (grid.y = token);
+    more go through the by-expert path.  Both must agree with the oracle and each other."""
+    s = H.Shape(1024, 512, 16, 4, router_mode=1, route_scale=2.5, clamp=10.0, seed=81)
+    x, logits, bias = H.host_inputs(s, T)
+    dw = H.device_weights(s)
+    layer = MoeLayer(dw, T)
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    layer.set_tuning(decode_max_tokens=8)
+    a, sel, w = layer.run(dx, dl, want_routing=True)
+    a = a.clone()
+    layer.set_tuning(decode_max_tokens=1)
+    b = layer.run(dx, None, selected_in=sel, weights_in=w)
+    torch.cuda.synchronize()
+    sel_h, w_h = sel.cpu().numpy(), w.cpu().numpy()
+    want = ref.moe_forward(H.host_weights(s, experts=np.unique(sel_h)), x, sel_h, w_h)
+    assert H.max_rel(a.cpu().numpy(), want) < OUT_TOL
+    assert H.max_rel(b.cpu().numpy(), want) < OUT_TOL
+    assert H.max_rel(a.cpu().numpy(), b.cpu().numpy()) < 1e-3
+    # an empty slot in the per-token path
+    sel2 = sel.clone()
+    sel2[T - 1, 1] = -1
+    layer.set_tuning(decode_max_tokens=8)
+    c = layer.run(dx, None, selected_in=sel2, weights_in=w)
+    sel2_h = sel2.cpu().numpy()
+    want2 = ref.moe_forward(H.host_weights(s, experts=np.unique(sel2_h[sel2_h >= 0])), x, sel2_h, w_h)
+    assert H.max_rel(c.cpu().numpy(), want2) < OUT_TOL
 
 
 @pytest.mark.parametrize("T", [1, 4, 16, 64])
