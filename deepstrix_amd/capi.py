@@ -54,6 +54,7 @@ SIGNATURES = {
     "dsx_last_error": (C.c_char_p, []),
     "dsx_init": (_int, []),
     "dsx_router_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _f32, _u32, _u32, _u32, _u32]),
+    "dsx_router_logits": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "dsx_q8k_quantize": (_int, [_vp, _vp, _vp, _u32]),
     "dsx_q8_0_quantize": (_int, [_vp, _vp, _vp, _vp, _u32]),
     "dsx_q8_0_quantize_rows": (_int, [_vp, _vp, _vp, _u32, _u32]),
@@ -77,6 +78,7 @@ SIGNATURES = {
     "dsx_moe_layer_set_profile_events": (_int, [_vp, _vp, _vp, _vp]),
     "dsx_moe_layer_set_tuning": (_int, [_vp, _u32, _u32, _u32]),
     "dsx_moe_layer_workspace_bytes": (_sz, [_vp, _u32]),
+    "dsx_moe_block_forward": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
     "dsx_moe_layer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _sz, _vp, _vp, _vp, _vp]),
 }
 

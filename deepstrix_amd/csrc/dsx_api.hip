@@ -284,7 +284,7 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
                             const uint8_t *xq, const int32_t *selected, const uint8_t *sh_down,
                             uint64_t dbpe, uint32_t xq_slot_stride, uint32_t n_used,
                             uint32_t n_rows, uint32_t n_blocks_in, bool staged = false,
-                            uint32_t n_tokens = 1) {
+                            uint32_t n_tokens = 1, const float *residual = nullptr) {
     if (!out || !down || !xq || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: null pointer");
     if (n_used > DSX_MAX_USED) return fail(DSX_ERR_INVALID_ARG, "moe_down_batched: n_used=%u", n_used);
@@ -309,6 +309,7 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     raise_lds_limits();
     DownDecodeParams p{};
     p.out = out; p.down = down; p.xq = xq; p.selected = selected; p.sh_down = sh_down;
+    p.residual = residual;
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.n_slots = n_slots;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
     if (staged)
@@ -487,6 +488,17 @@ static int reduce_impl(hipStream_t st, float *out, const float *partials, const 
 int dsx_moe_reduce_partials(dsx_stream_t stream, float *out, const float *partials,
                             const int32_t *selected, uint32_t n_used, uint32_t n_rows, uint32_t b) {
     return reduce_impl(S(stream), out, partials, selected, nullptr, n_used, n_rows, b);
+}
+
+int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w, const float *x,
+                      uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
+    if (n_tokens == 0) return DSX_OK;
+    if (!logits || !router_w || !x) return fail(DSX_ERR_INVALID_ARG, "router_logits: null pointer");
+    if (n_expert == 0 || hidden == 0) return fail(DSX_ERR_INVALID_ARG, "router_logits: n_expert=%u hidden=%u", n_expert, hidden);
+    hipLaunchKernelGGL(k_router_logits<false>, dim3(n_expert), dim3(256), 0, S(stream), logits,
+                       (float *)nullptr, router_w, x, (const float *)nullptr, 0.0f, n_expert, hidden,
+                       n_tokens);
+    return launched("router_logits");
 }
 
 // ---- element-wise -----------------------------------------------------------------------

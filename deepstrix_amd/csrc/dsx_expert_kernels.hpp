@@ -314,6 +314,7 @@ struct DownDecodeParams {
     const uint8_t *xq;      // slot-major activation rows (Q8_K or staged), xq_slot_stride apart
     const int32_t *selected;  // [n_tokens, n_used]
     const uint8_t *sh_down;   // extra slot n_used, or null
+    const float *residual;    // [n_tokens, n_rows] added to the result (may alias out), or null
     uint64_t dbpe;
     uint32_t xq_slot_stride, n_used, n_slots, n_rows, n_blocks_in;
 };
@@ -400,6 +401,7 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
         float s = 0.0f;
 #pragma unroll
         for (int wv = 0; wv < kDownWaves; wv++) s += s_red[wv][i][l];
+        if (p.residual) s += p.residual[(uint64_t)blockIdx.y * p.n_rows + row0 + tid];
         out[row0 + tid] = s;
     }
 }

@@ -572,6 +572,99 @@ __global__ __launch_bounds__(256) void k_rms_norm(float *__restrict__ out,
     for (uint32_t i = tid; i < n; i += 256u) orow[i] = xr[i] * scale * weight[i];
 }
 
+// Router logits logits[t, e] = sum_k W[e, k] * x[t, k] in f32, one workgroup per expert, up
+// to kRlTokens tokens per pass (crates/v4flash-kernels/kernels/laguna_ops.hip:57-60; the
+// engine's f32 router matvec, crates/v4flash-kernels/src/het/forward_prefill.rs:8974-9015).
+// NORM: x is first RMS-normalized (same arithmetic as k_rms_norm) and the workgroups with
+// e < n_tokens also write the normalized row e to xn, so one launch replaces the norm, the
+// router matvec and the copy between them.
+constexpr int kRlTokens = 4;
+
+template <bool NORM>
+__global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logits,
+                                                       float *__restrict__ xn,
+                                                       const float *__restrict__ w,
+                                                       const float *__restrict__ x,
+                                                       const float *__restrict__ norm_w, float eps,
+                                                       uint32_t n_expert, uint32_t hidden,
+                                                       uint32_t n_tokens) {
+    __shared__ float sdata[256];
+    __shared__ float s_scale[kRlTokens];
+    __shared__ float s_part[4][kRlTokens];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t e = blockIdx.x;
+    const float *wr = w + (uint64_t)e * hidden;
+    for (uint32_t t0 = 0; t0 < n_tokens; t0 += kRlTokens) {
+        const uint32_t nt = min((uint32_t)kRlTokens, n_tokens - t0);
+        if (NORM) {
+            for (uint32_t j = 0; j < nt; j++) {
+                const float *xr = x + (uint64_t)(t0 + j) * hidden;
+                double partial = 0.0;
+                for (uint32_t i = tid; i < hidden; i += 256u) {
+                    const float v = xr[i];
+                    partial += (double)v * (double)v;
+                }
+                sdata[tid] = (float)partial;
+                __syncthreads();
+                for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+                    if (tid < stride) sdata[tid] += sdata[tid + stride];
+                    __syncthreads();
+                }
+                if (tid == 0) s_scale[j] = 1.0f / sqrtf(sdata[0] / (float)hidden + eps);
+                __syncthreads();
+            }
+        }
+        float acc[kRlTokens];
+#pragma unroll
+        for (int j = 0; j < kRlTokens; j++) acc[j] = 0.0f;
+        for (uint32_t i = tid; i < hidden; i += 256u) {
+            const float wv = wr[i];
+            const float nw = NORM ? norm_w[i] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < kRlTokens; j++) {
+                if ((uint32_t)j < nt) {
+                    float xv = x[(uint64_t)(t0 + j) * hidden + i];
+                    if (NORM) {
+                        xv = xv * s_scale[j] * nw;
+                        if (e == t0 + j) xn[(uint64_t)(t0 + j) * hidden + i] = xv;
+                    }
+                    acc[j] = fmaf(wv, xv, acc[j]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kRlTokens; j++) {
+            const float v = wave_sum_f32(acc[j]);
+            if (lane == 0) s_part[wave][j] = v;
+        }
+        __syncthreads();
+        if (tid < nt)
+            logits[(uint64_t)(t0 + tid) * n_expert + e] =
+                s_part[0][tid] + s_part[1][tid] + s_part[2][tid] + s_part[3][tid];
+        __syncthreads();
+    }
+    // rows whose index has no workgroup (n_tokens > n_expert): written by workgroup 0
+    if (NORM && e == 0 && n_tokens > n_expert) {
+        for (uint32_t t = n_expert; t < n_tokens; t++) {
+            const float *xr = x + (uint64_t)t * hidden;
+            double partial = 0.0;
+            for (uint32_t i = tid; i < hidden; i += 256u) {
+                const float v = xr[i];
+                partial += (double)v * (double)v;
+            }
+            sdata[tid] = (float)partial;
+            __syncthreads();
+            for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+                if (tid < stride) sdata[tid] += sdata[tid + stride];
+                __syncthreads();
+            }
+            const float scale = 1.0f / sqrtf(sdata[0] / (float)hidden + eps);
+            __syncthreads();
+            for (uint32_t i = tid; i < hidden; i += 256u) xn[(uint64_t)t * hidden + i] = xr[i] * scale * norm_w[i];
+        }
+    }
+}
+
 // HF packed nibbles + E8M0 scales -> v2 super-block rows, one thread per 32-element block.
 // crates/v4flash-kernels/kernels/mxfp4_repack.hip:35-65 (same bytes as
 // crates/v4flash-core/src/hf_v41.rs:1208-1232).

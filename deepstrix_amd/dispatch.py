@@ -46,6 +46,13 @@ def router_topk(selected, weights, logits, bias, n_expert, n_used, scale, eps, b
                                 n_expert, n_used, scale, eps, b, mode, n_group, topk_group))
 
 
+def router_logits(logits, router_w, x, n_expert, hidden, n_tokens):
+    """crates/v4flash-kernels/kernels/laguna_ops.hip:57-60 (f32 W . x)"""
+    capi.init()
+    check(lib().dsx_router_logits(_stream(), _p(logits), _p(router_w), _p(x), n_expert, hidden,
+                                  n_tokens))
+
+
 def q8k_quantize(out, x, n_blocks):
     capi.init()
     check(lib().dsx_q8k_quantize(_stream(), _p(out), _p(x), n_blocks))

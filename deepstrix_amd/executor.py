@@ -45,6 +45,10 @@ class LayerWeights:
     sh_up_fmt: int = FMT_MXFP4
     sh_down_fmt: int = FMT_MXFP4
     sh_clamp: float = 0.0
+    # pre-norm block (chained layers): RMSNorm weight [hidden], router matrix f32 [n_expert, hidden]
+    norm_w: Optional[torch.Tensor] = None
+    norm_eps: float = 1e-6
+    router_w: Optional[torch.Tensor] = None
 
 
 class MoeLayer:
@@ -99,6 +103,20 @@ class MoeLayer:
         check(lib().dsx_moe_layer_set_tuning(self._h, by_expert_chunk, gemm_min_tokens,
                                              decode_max_tokens))
 
+    def block(self, h: torch.Tensor) -> torch.Tensor:
+        """In place: h += layer(RMSNorm(h)), router logits = router_w . RMSNorm(h)
+        (include/dsx_moe.h: dsx_moe_block_forward)."""
+        T = h.shape[0]
+        if T > self.max_tokens:
+            raise ValueError(f"{T} tokens > max_tokens={self.max_tokens}")
+        w = self.w
+        if w.norm_w is None or w.router_w is None:
+            raise ValueError("block() needs norm_w and router_w")
+        check(lib().dsx_moe_block_forward(
+            self._h, torch.cuda.current_stream().cuda_stream, h.data_ptr(), w.norm_w.data_ptr(),
+            w.norm_eps, w.router_w.data_ptr(), T, self.workspace.data_ptr(), self.workspace_bytes))
+        return h
+
     def run(self, x: torch.Tensor, logits: Optional[torch.Tensor] = None, out=None,
             selected_in=None, weights_in=None, want_routing=False):
         """x f32 [T, hidden], logits f32 [T, n_expert] -> out f32 [T, hidden]."""
@@ -120,3 +138,45 @@ class MoeLayer:
         if want_routing:
             return out, sel_out, w_out
         return out
+
+
+class MoeChain:
+    """A stack of pre-norm residual MoE blocks run back to back on one stream, optionally
+    replayed from a HIP graph (launch-bound at small token counts).  The counterpart of the
+    reference's per-layer loop around `issue_igpu_moe`
+    (crates/v4flash-kernels/src/het/forward_layer.rs:424-466)."""
+
+    def __init__(self, weights, max_tokens: int):
+        self.layers = [MoeLayer(w, max_tokens) for w in weights]
+        self.max_tokens = max_tokens
+        self._graph = None
+        self._static_h = None
+
+    def step(self, h: torch.Tensor) -> torch.Tensor:
+        """In place over all layers."""
+        for layer in self.layers:
+            layer.block(h)
+        return h
+
+    def capture(self, n_tokens: int) -> None:
+        """Records one step for `n_tokens` tokens into a graph; `replay` then runs it."""
+        hidden = self.layers[0].w.hidden
+        self._static_h = torch.zeros((n_tokens, hidden), dtype=torch.float32, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):   # warm-up outside the capture
+            self.step(self._static_h)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self._static_h.zero_()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.step(self._static_h)
+        self._graph = g
+
+    def replay(self, h: torch.Tensor) -> torch.Tensor:
+        """One captured step on a copy of h; returns the graph's output buffer (valid until
+        the next replay)."""
+        self._static_h.copy_(h)
+        self._graph.replay()
+        return self._static_h

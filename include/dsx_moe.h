@@ -78,6 +78,12 @@ int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, cons
                     const float *bias, uint32_t n_expert, uint32_t n_used, float scale, float eps,
                     uint32_t b, uint32_t mode, uint32_t n_group, uint32_t topk_group);
 
+/* f32 router matvec: logits[t,e] = sum_k router_w[e,k] * x[t,k]
+ * (crates/v4flash-kernels/kernels/laguna_ops.hip:57-60;
+ * crates/v4flash-kernels/src/het/forward_prefill.rs:8974-9015). */
+int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w, const float *x,
+                      uint32_t n_expert, uint32_t hidden, uint32_t n_tokens);
+
 /* ---- activation quantizers ------------------------------------------------
  * Q8KQuantize::launch (crates/v4flash-kernels/src/q8_k.rs:33-104). */
 int dsx_q8k_quantize(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t n_blocks);
@@ -227,6 +233,17 @@ int dsx_moe_layer_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
                           const float *logits, uint32_t n_tokens, void *workspace,
                           size_t workspace_bytes, int32_t *selected_out, float *weights_out,
                           const int32_t *selected_in, const float *weights_in);
+
+/* One pre-norm residual MoE block (the unit of BASELINE's chained-layer decode):
+ *   h[t,:] += layer(RMSNorm(h[t,:]; norm_w, eps)),  router logits = router_w . RMSNorm(h[t,:])
+ * RMSNorm as crates/v4flash-kernels/kernels/rms_norm.hip:12-50, the f32 router matvec as
+ * crates/v4flash-kernels/src/het/forward_prefill.rs:8974-9015, the residual add as
+ * kernels/vec_add.hip:6-13; sequencing of crates/v4flash-kernels/src/het/forward_layer.rs:424-466.
+ * h is f32 [n_tokens, hidden], updated in place; router_w f32 [n_expert, hidden];
+ * norm_w f32 [hidden].  Same workspace as dsx_moe_layer_forward. */
+int dsx_moe_block_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *h, const float *norm_w,
+                          float eps, const float *router_w, uint32_t n_tokens, void *workspace,
+                          size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

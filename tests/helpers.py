@@ -90,7 +90,7 @@ def host_inputs(s: Shape, T: int, logit_shift: Optional[np.ndarray] = None):
     return x, logits, bias
 
 
-def device_weights(s: Shape, device="cuda"):
+def device_weights(s: Shape, device="cuda", block=False):
     """The same layer generated on the GPU (identical bytes)."""
     import torch
     from deepstrix_amd.executor import LayerWeights
@@ -110,8 +110,20 @@ def device_weights(s: Shape, device="cuda"):
         w.sh_gate_fmt = w.sh_up_fmt = s.shg
         w.sh_down_fmt = s.shd
         w.sh_clamp = s.clamp
+    if block:
+        w.norm_w = synth.normal_dev(s.seed, synth.T_NORM_W, s.hidden, 0.02, 1.0)
+        w.router_w = synth.normal_dev(s.seed, synth.T_ROUTER_W, s.n_expert * s.hidden, 0.02)
+        w.norm_eps = 1e-6
     torch.cuda.synchronize()
     return w
+
+
+def host_block_params(s: Shape):
+    """RMSNorm weight 1 + N(0, 0.02) and router matrix N(0, 0.02) of a pre-norm block
+    (BASELINE config 4), the same values device_weights(block=True) generates."""
+    norm_w = synth.normal_host(s.seed, synth.T_NORM_W, s.hidden, 0.02, 1.0)
+    router_w = synth.normal_host(s.seed, synth.T_ROUTER_W, s.n_expert * s.hidden, 0.02)
+    return norm_w, router_w.reshape(s.n_expert, s.hidden)
 
 
 def oracle_route(s: Shape, logits, bias):

@@ -1,0 +1,126 @@
+"""GPU parity of the pre-norm residual MoE block and of chained blocks (BASELINE config 4:
+stacked layers with RMSNorm + residual, 2 tokens per step), eager and replayed from a graph."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from deepstrix_amd import dispatch
+from deepstrix_amd.executor import MoeChain, MoeLayer
+from oracle import ref
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 2e-3
+
+
+def oracle_block(s, h, experts_cache=None):
+    """h + layer(RMSNorm(h)) on the CPU; also the smallest k/(k+1) score gap per token."""
+    norm_w, router_w = H.host_block_params(s)
+    xn = ref.rms_norm(h, norm_w, 1e-6)
+    logits = ref.router_logits(router_w, xn)
+    bias = None
+    if s.bias_sigma:
+        _, _, bias = H.host_inputs(s, 1)
+    sel, w = H.oracle_route(s, logits, bias)
+    _, scores = ref.router_scores(logits, bias, s.router_mode, s.n_group, s.topk_group)
+    gaps = []
+    for t in range(h.shape[0]):
+        sc = np.sort(scores[t][np.isfinite(scores[t])])[::-1]
+        gaps.append(float(sc[s.n_used - 1] - sc[s.n_used]))
+    hw = H.host_weights(s, experts=np.unique(sel))
+    out = ref.moe_forward(hw, xn, sel, w)
+    return (h + out).astype(np.float32), xn, logits, np.array(gaps)
+
+
+def layer_shapes(base, n):
+    return [H.Shape(**{**base.__dict__, "seed": base.seed + 0x100 * i}) for i in range(n)]
+
+
+def test_router_logits_operator():
+    rng = np.random.default_rng(0)
+    for T, E, hidden in [(1, 64, 2048), (5, 256, 7168), (9, 16, 520)]:
+        W = rng.normal(0, 0.02, (E, hidden)).astype(np.float32)
+        x = rng.normal(0, 1, (T, hidden)).astype(np.float32)
+        out = torch.zeros((T, E), dtype=torch.float32, device="cuda")
+        dispatch.router_logits(out, torch.from_numpy(W).cuda(), torch.from_numpy(x).cuda(), E, hidden, T)
+        np.testing.assert_allclose(out.cpu().numpy(), ref.router_logits(W, x), atol=3e-5)
+
+
+@pytest.mark.parametrize("T", [1, 2, 4, 6, 130])
+def test_block_matches_oracle(T):
+    """decode path (residual fused into `down`), by-expert path and GEMM path."""
+    s = H.Shape(1024, 512, 16, 4, router_mode=1, n_group=4, topk_group=2, route_scale=2.5,
+                bias_sigma=0.01, clamp=10.0, seed=101)
+    dw = H.device_weights(s, block=True)
+    layer = MoeLayer(dw, T)
+    h, _, _ = H.host_inputs(s, T)
+    h = (h * 1.7).astype(np.float32)
+    want, xn, logits, gaps = oracle_block(s, h)
+    dh = torch.from_numpy(h).cuda()
+    layer.block(dh)
+    got = dh.cpu().numpy()
+    ok = gaps > 1e-4
+    assert ok.mean() > 0.9
+    assert H.max_rel(got[ok] - h[ok], want[ok] - h[ok]) < OUT_TOL   # the layer's contribution
+    assert H.max_rel(got[ok], want[ok]) < OUT_TOL
+
+
+def run_chain_oracle(shapes, h):
+    min_gap = np.inf
+    for s in shapes:
+        h, _, _, gaps = oracle_block(s, h)
+        min_gap = min(min_gap, gaps.min())
+    return h, min_gap
+
+
+def test_small_chain_eager_and_graph():
+    base = H.Shape(512, 256, 8, 2, router_mode=1, route_scale=2.5, clamp=10.0, seed=111)
+    shapes = layer_shapes(base, 3)
+    chain = MoeChain([H.device_weights(s, block=True) for s in shapes], 2)
+    rng = np.random.default_rng(1)
+    chain.capture(2)
+    for step in range(4):   # fresh inputs each step; eager work between the replays
+        h = rng.normal(0, 1, (2, base.hidden)).astype(np.float32)
+        want, min_gap = run_chain_oracle(shapes, h)
+        eager = chain.step(torch.from_numpy(h).cuda()).clone()
+        torch.cuda.synchronize()
+        replayed = chain.replay(torch.from_numpy(h).cuda()).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(eager, replayed), f"graph replay {step} differs from the eager step"
+        if min_gap > 1e-2:   # every pick decided by a margin far above the f32 noise carried along
+            assert H.max_rel(eager.cpu().numpy(), want) < 3 * OUT_TOL   # three layers deep
+
+
+def test_config4_chain_of_v3_layers():
+    """8 chained V3-shape MXFP4 layers, RMSNorm eps 1e-6 + residual, T = 2."""
+    shapes = layer_shapes(H.CFG2, 8)
+    chain = MoeChain([H.device_weights(s, block=True) for s in shapes], 2)
+    rng = np.random.default_rng(4)
+    h = rng.normal(0, 1, (2, H.CFG2.hidden)).astype(np.float32)
+    # layer by layer on the oracle's running state, so that one near-tie cannot hide the rest
+    cur = h
+    checked = 0
+    for i, s in enumerate(shapes):
+        want, _, _, gaps = oracle_block(s, cur)
+        dh = torch.from_numpy(cur).cuda()
+        chain.layers[i].block(dh)
+        got = dh.cpu().numpy()
+        ok = gaps > 1e-4
+        if ok.any():
+            assert H.max_rel(got[ok] - cur[ok], want[ok] - cur[ok]) < OUT_TOL, f"layer {i}"
+            checked += int(ok.sum())
+        cur = want
+    assert checked >= 12
+    chain.capture(2)
+    eager = chain.step(torch.from_numpy(h).cuda()).clone()
+    for _ in range(3):
+        replayed = chain.replay(torch.from_numpy(h).cuda()).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(eager, replayed)
+    # End to end the state carries each layer's f32-level differences into the next router, so
+    # the whole chain is only comparable when every pick is decided by a comfortable margin.
+    want_all, min_gap = run_chain_oracle(shapes, h)
+    if min_gap > 1e-2:
+        assert H.max_rel(eager.cpu().numpy(), want_all) < 8 * OUT_TOL
