@@ -117,6 +117,46 @@ def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
             "mfma_frac_useful_vs_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK}
 
 
+def chain_leg(H, torch, np, n_layers=8, T=2, steps=256):
+    """BASELINE config 4: 8 chained V3-shape MXFP4 layers, each h += MoE(RMSNorm(h)), T = 2
+    tokens per step, 256 consecutive steps with fresh N(0,1) inputs.  Latency of one step from
+    the host's point of view (submit + run + synchronize), eager and replayed from a graph."""
+    from deepstrix_amd.executor import MoeChain
+    shapes = [H.Shape(**{**H.CFG2.__dict__, "seed": H.CFG2.seed + 0x1000 + 0x100 * i}) for i in range(n_layers)]
+    chain = MoeChain([H.device_weights(s, block=True) for s in shapes], T)
+    hidden = H.CFG2.hidden
+    inputs = torch.randn((steps, T, hidden), dtype=torch.float32, device="cuda",
+                         generator=torch.Generator(device="cuda").manual_seed(4))
+    h = torch.empty((T, hidden), dtype=torch.float32, device="cuda")
+
+    def timed(fn):
+        for i in range(8):
+            fn(inputs[i])
+        torch.cuda.synchronize()
+        lat = np.empty(steps)
+        for i in range(steps):
+            t0 = time.perf_counter()
+            fn(inputs[i])
+            torch.cuda.synchronize()
+            lat[i] = (time.perf_counter() - t0) * 1e6
+        return lat
+
+    def eager(x):
+        h.copy_(x)
+        chain.step(h)
+
+    lat_e = timed(eager)
+    chain.capture(T)
+    lat_g = timed(chain.replay)
+    q = lambda a: {"p10": float(np.percentile(a, 10)), "p50": float(np.percentile(a, 50)),
+                   "p90": float(np.percentile(a, 90))}
+    per_step_bytes = n_layers * T * 9 * EXPERT_BYTES
+    return {"layers": n_layers, "tokens_per_step": T, "steps": steps,
+            "eager_us_per_step": q(lat_e), "graph_us_per_step": q(lat_g),
+            "launches_per_step": n_layers * 4,
+            "graph_GBps_p50": per_step_bytes / (np.percentile(lat_g, 50) * 1e-6) / 1e9}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,6 +165,7 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="independent layers the steps rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the T=4096 prefill leg")
+    ap.add_argument("--no-chain", action="store_true", help="skip the 8-layer chained decode leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -217,6 +258,8 @@ def main():
 
     if not args.no_prefill:
         extra["prefill_T4096"] = prefill_leg(layers[0].w, base, H, torch, np)
+    if not args.no_chain:
+        extra["chain_8_layers_T2"] = chain_leg(H, torch, np)
 
     result = {
         "metric": "moe_layer_us_per_token_T1",
