@@ -495,6 +495,8 @@ int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w,
     if (n_tokens == 0) return DSX_OK;
     if (!logits || !router_w || !x) return fail(DSX_ERR_INVALID_ARG, "router_logits: null pointer");
     if (n_expert == 0 || hidden == 0) return fail(DSX_ERR_INVALID_ARG, "router_logits: n_expert=%u hidden=%u", n_expert, hidden);
+    if (!aligned(router_w, 16) || !aligned(x, 16))
+        return fail(DSX_ERR_SHAPE, "router_logits: router_w and x must be 16-byte aligned");
     hipLaunchKernelGGL(k_router_logits<false>, dim3(n_expert), dim3(256), 0, S(stream), logits,
                        (float *)nullptr, router_w, x, (const float *)nullptr, 0.0f, n_expert, hidden,
                        n_tokens);

@@ -580,6 +580,15 @@ __global__ __launch_bounds__(256) void k_rms_norm(float *__restrict__ out,
 // router matvec and the copy between them.
 constexpr int kRlTokens = 4;
 
+// Sum over the 256 threads of a workgroup; every thread gets the result.  `red` holds 4 floats.
+__device__ __forceinline__ float block_sum_256(float v, float *red, uint32_t tid) {
+    v = wave_sum_f32(v);
+    __syncthreads();  // `red` may still be read from a previous call
+    if ((tid & 63u) == 0u) red[tid >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
 template <bool NORM>
 __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logits,
                                                        float *__restrict__ xn,
@@ -588,44 +597,65 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
                                                        const float *__restrict__ norm_w, float eps,
                                                        uint32_t n_expert, uint32_t hidden,
                                                        uint32_t n_tokens) {
-    __shared__ float sdata[256];
-    __shared__ float s_scale[kRlTokens];
-    __shared__ float s_part[4][kRlTokens];
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    __shared__ float s_red[4];
+    const uint32_t tid = threadIdx.x;
     const uint32_t e = blockIdx.x;
     const float *wr = w + (uint64_t)e * hidden;
+    // float4 loads need 16-byte aligned rows; otherwise everything goes one element at a time
+    const uint32_t n4 = (hidden % 4u == 0u) ? hidden / 4u : 0u;
     for (uint32_t t0 = 0; t0 < n_tokens; t0 += kRlTokens) {
         const uint32_t nt = min((uint32_t)kRlTokens, n_tokens - t0);
-        if (NORM) {
-            for (uint32_t j = 0; j < nt; j++) {
+        float scale[kRlTokens];
+#pragma unroll
+        for (int j = 0; j < kRlTokens; j++) {
+            scale[j] = 1.0f;
+            if (NORM && (uint32_t)j < nt) {
+                // mean of squares with f64 partial sums, like k_rms_norm
                 const float *xr = x + (uint64_t)(t0 + j) * hidden;
                 double partial = 0.0;
-                for (uint32_t i = tid; i < hidden; i += 256u) {
-                    const float v = xr[i];
-                    partial += (double)v * (double)v;
+                for (uint32_t i = tid; i < n4; i += 256u) {
+                    const float4 v = *(const float4 *)(xr + 4u * i);
+                    partial += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
                 }
-                sdata[tid] = (float)partial;
-                __syncthreads();
-                for (uint32_t stride = 128; stride > 0; stride >>= 1) {
-                    if (tid < stride) sdata[tid] += sdata[tid + stride];
-                    __syncthreads();
-                }
-                if (tid == 0) s_scale[j] = 1.0f / sqrtf(sdata[0] / (float)hidden + eps);
-                __syncthreads();
+                for (uint32_t i = 4u * n4 + tid; i < hidden; i += 256u) partial += (double)xr[i] * xr[i];
+                const float ss = block_sum_256((float)partial, s_red, tid);
+                scale[j] = 1.0f / sqrtf(ss / (float)hidden + eps);
             }
         }
         float acc[kRlTokens];
 #pragma unroll
         for (int j = 0; j < kRlTokens; j++) acc[j] = 0.0f;
-        for (uint32_t i = tid; i < hidden; i += 256u) {
+        for (uint32_t i = tid; i < n4; i += 256u) {
+            const float4 wv = *(const float4 *)(wr + 4u * i);
+            float4 nw = {1.f, 1.f, 1.f, 1.f};
+            if (NORM) nw = *(const float4 *)(norm_w + 4u * i);
+#pragma unroll
+            for (int j = 0; j < kRlTokens; j++) {
+                if ((uint32_t)j < nt) {
+                    float4 xv = *(const float4 *)(x + (uint64_t)(t0 + j) * hidden + 4u * i);
+                    if (NORM) {
+                        xv.x = xv.x * scale[j] * nw.x;
+                        xv.y = xv.y * scale[j] * nw.y;
+                        xv.z = xv.z * scale[j] * nw.z;
+                        xv.w = xv.w * scale[j] * nw.w;
+                        if (e == t0 + j)
+                            *(float4 *)(xn + (uint64_t)(t0 + j) * hidden + 4u * i) = xv;
+                    }
+                    acc[j] = fmaf(wv.x, xv.x, acc[j]);
+                    acc[j] = fmaf(wv.y, xv.y, acc[j]);
+                    acc[j] = fmaf(wv.z, xv.z, acc[j]);
+                    acc[j] = fmaf(wv.w, xv.w, acc[j]);
+                }
+            }
+        }
+        for (uint32_t i = 4u * n4 + tid; i < hidden; i += 256u) {
             const float wv = wr[i];
-            const float nw = NORM ? norm_w[i] : 1.0f;
 #pragma unroll
             for (int j = 0; j < kRlTokens; j++) {
                 if ((uint32_t)j < nt) {
                     float xv = x[(uint64_t)(t0 + j) * hidden + i];
                     if (NORM) {
-                        xv = xv * s_scale[j] * nw;
+                        xv = xv * scale[j] * norm_w[i];
                         if (e == t0 + j) xn[(uint64_t)(t0 + j) * hidden + i] = xv;
                     }
                     acc[j] = fmaf(wv, xv, acc[j]);
@@ -634,33 +664,21 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
         }
 #pragma unroll
         for (int j = 0; j < kRlTokens; j++) {
-            const float v = wave_sum_f32(acc[j]);
-            if (lane == 0) s_part[wave][j] = v;
+            if ((uint32_t)j < nt) {
+                const float v = block_sum_256(acc[j], s_red, tid);
+                if (tid == 0) logits[(uint64_t)(t0 + j) * n_expert + e] = v;
+            }
         }
-        __syncthreads();
-        if (tid < nt)
-            logits[(uint64_t)(t0 + tid) * n_expert + e] =
-                s_part[0][tid] + s_part[1][tid] + s_part[2][tid] + s_part[3][tid];
-        __syncthreads();
     }
-    // rows whose index has no workgroup (n_tokens > n_expert): written by workgroup 0
+    // normalized rows whose index has no workgroup (n_tokens > n_expert): workgroup 0 writes them
     if (NORM && e == 0 && n_tokens > n_expert) {
         for (uint32_t t = n_expert; t < n_tokens; t++) {
             const float *xr = x + (uint64_t)t * hidden;
             double partial = 0.0;
-            for (uint32_t i = tid; i < hidden; i += 256u) {
-                const float v = xr[i];
-                partial += (double)v * (double)v;
-            }
-            sdata[tid] = (float)partial;
-            __syncthreads();
-            for (uint32_t stride = 128; stride > 0; stride >>= 1) {
-                if (tid < stride) sdata[tid] += sdata[tid + stride];
-                __syncthreads();
-            }
-            const float scale = 1.0f / sqrtf(sdata[0] / (float)hidden + eps);
-            __syncthreads();
-            for (uint32_t i = tid; i < hidden; i += 256u) xn[(uint64_t)t * hidden + i] = xr[i] * scale * norm_w[i];
+            for (uint32_t i = tid; i < hidden; i += 256u) partial += (double)xr[i] * xr[i];
+            const float ss = block_sum_256((float)partial, s_red, tid);
+            const float sc = 1.0f / sqrtf(ss / (float)hidden + eps);
+            for (uint32_t i = tid; i < hidden; i += 256u) xn[(uint64_t)t * hidden + i] = xr[i] * sc * norm_w[i];
         }
     }
 }
