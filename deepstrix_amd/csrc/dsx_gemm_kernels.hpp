@@ -78,11 +78,16 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t g4 = lane >> 4, n16 = lane & 15u;
 
-    // Workgroups are dealt to the 8 XCDs round-robin by id.  All row tiles of one work item
-    // go to the same XCD one after another, so the item's activations are fetched into one
-    // L2 only, and the row tiles of the next item of that XCD follow.
+    // Workgroups are dealt to the 8 XCDs round-robin by id, and each XCD has its own L2.  An
+    // XCD gets a contiguous range of work items; its 32 concurrent workgroups are then four
+    // consecutive items (usually column tiles of the same expert: they stream the same weights
+    // in step) times the eight row tiles of each (they stream the same activations).
     const uint32_t xcd = blockIdx.x & 7u, seq = blockIdx.x >> 3;
-    const uint32_t item = xcd + 8u * (seq / p.n_row_tiles);
+    const uint32_t n_items = (uint32_t)*p.n_work_items;   // the grid is only an upper bound
+    const uint32_t items_per_xcd = (n_items + 7u) / 8u;
+    const uint32_t local = seq / p.n_row_tiles;
+    if (local >= items_per_xcd) return;
+    const uint32_t item = xcd * items_per_xcd + local;
     const uint32_t rt = seq % p.n_row_tiles;
     if ((int)item >= *p.n_work_items) return;  // uniform: the grid is an upper bound
 
@@ -175,6 +180,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
 #pragma unroll
             for (int j = 0; j < 4; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
+    const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
     for (uint32_t sb = 0; sb < p.n_sb; sb++) {
         const uint32_t buf = sb & 1u;
         const bool more = sb + 1u < p.n_sb;
@@ -183,72 +189,74 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
             load_a(a_nxt, sb + 1u);
         }
         const uint8_t *tile = tiles + buf * kGemmTileBytes;
+        // A column group j (16 columns) needs four B pieces: (half 0, high plane), (half 0, low),
+        // (half 1, high), (half 1, low).  Piece p of group j lives in chunk rows 2p and 2p + 1:
+        // chunk row i = ((h * 2 + plane) * 2 + c) * 4 + kb, 64 columns of 16 bytes each.
+        // The pieces are walked in order with the next one already loading while the eight
+        // fragments' instructions of the current one issue; the fold of group j - 1 into the
+        // accumulators (acc += d * c) is interleaved with the first piece of group j, right
+        // before each fragment's temporary is overwritten.
+        constexpr uint32_t CR = 4u * kGemmMT * 16u;  // one (h, plane, c) step
+        auto load_piece = [&](int j, int pc) -> v8i {
+            const uint32_t cb = (g4 * kGemmMT + (uint32_t)j * 16u + n16) * 16u;
+            return b_operand(tile, cb + (2u * pc) * CR, cb + (2u * pc + 1u) * CR);
+        };
+        v4f c[kGemmRF][2];
+        v8i bq = load_piece(0, 0);
+        float yd_prev = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            if ((uint32_t)j * 16u >= cnt) break;  // uniform: no column of this group is real
-            // chunk row i = ((h * 2 + plane) * 2 + c) * 4 + kb, 64 columns of 16 bytes each
-            const uint32_t cb = (g4 * kGemmMT + j * 16u + n16) * 16u;
-            constexpr uint32_t CR = 4u * kGemmMT * 16u;  // one (h, plane, c) step
-            const v8i h0 = b_operand(tile, cb + 0u * CR, cb + 1u * CR);
-            const v8i l0 = b_operand(tile, cb + 2u * CR, cb + 3u * CR);
-            const v8i h1 = b_operand(tile, cb + 4u * CR, cb + 5u * CR);
-            const v8i l1 = b_operand(tile, cb + 6u * CR, cb + 7u * CR);
-            const float yd = s_yd[buf * kGemmMT + j * 16u + n16];
-            v4f c[kGemmRF][2];
+            if ((uint32_t)j < nj) {  // uniform
+                const float yd = s_yd[buf * kGemmMT + j * 16u + n16];
 #pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
+                for (int pc = 0; pc < 4; pc++) {
+                    v8i bn = bq;
+                    if (pc < 3) bn = load_piece(j, pc + 1);
+                    else if (j < 3 && (uint32_t)(j + 1) < nj) bn = load_piece(j + 1, 0);
 #pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    const WSuper &w = a_cur.f[r][m];
-                    const v8i a0 = {(int)w.a0.x, (int)w.a0.y, (int)w.a0.z, (int)w.a0.w, 0, 0, 0, 0};
-                    const int s0 = (int)((w.s.x >> (g4 * 8u)) & 0xFFu);
-                    c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        a0, h0, v4f{0.f, 0.f, 0.f, 0.f}, 4, 0, 0, s0, 0, 131);
+                    for (int r = 0; r < kGemmRF; r++)
+#pragma unroll
+                        for (int m = 0; m < 2; m++) {
+                            const WSuper &w = a_cur.f[r][m];
+                            const U4A8 &aw = pc < 2 ? w.a0 : w.a1;
+                            const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
+                            const int sc = (int)(((pc < 2 ? w.s.x : w.s.y) >> (g4 * 8u)) & 0xFFu);
+                            if (pc == 0) {
+                                if (j > 0) {
+                                    acc[r][m][j > 0 ? j - 1 : 0].x = fmaf(yd_prev, c[r][m].x, acc[r][m][j > 0 ? j - 1 : 0].x);
+                                    acc[r][m][j > 0 ? j - 1 : 0].y = fmaf(yd_prev, c[r][m].y, acc[r][m][j > 0 ? j - 1 : 0].y);
+                                    acc[r][m][j > 0 ? j - 1 : 0].z = fmaf(yd_prev, c[r][m].z, acc[r][m][j > 0 ? j - 1 : 0].z);
+                                    acc[r][m][j > 0 ? j - 1 : 0].w = fmaf(yd_prev, c[r][m].w, acc[r][m][j > 0 ? j - 1 : 0].w);
+                                }
+                                c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                    av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 0, 0, sc, 0, 131);
+                            } else {
+                                c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                    av, bq, c[r][m], 4, 0, 0, sc, 0, (pc & 1) ? 127 : 131);
+                            }
+                        }
+                    bq = bn;
                 }
-#pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    const WSuper &w = a_cur.f[r][m];
-                    const v8i a0 = {(int)w.a0.x, (int)w.a0.y, (int)w.a0.z, (int)w.a0.w, 0, 0, 0, 0};
-                    const int s0 = (int)((w.s.x >> (g4 * 8u)) & 0xFFu);
-                    c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a0, l0, c[r][m], 4, 0, 0,
-                                                                               s0, 0, 127);
+                yd_prev = yd;
+                if (j == 1 && more) {  // second half of the next tile's staging
+                    stage_store(buf ^ 1u, 0);
+                    stage_load(sb + 1u, 1);
                 }
+            }
+        }
+        // fold the last group
 #pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
+        for (int j = 0; j < 4; j++) {
+            if ((uint32_t)j + 1u == nj) {
 #pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    const WSuper &w = a_cur.f[r][m];
-                    const v8i a1 = {(int)w.a1.x, (int)w.a1.y, (int)w.a1.z, (int)w.a1.w, 0, 0, 0, 0};
-                    const int s1 = (int)((w.s.y >> (g4 * 8u)) & 0xFFu);
-                    c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a1, h1, c[r][m], 4, 0, 0,
-                                                                               s1, 0, 131);
-                }
+                for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    const WSuper &w = a_cur.f[r][m];
-                    const v8i a1 = {(int)w.a1.x, (int)w.a1.y, (int)w.a1.z, (int)w.a1.w, 0, 0, 0, 0};
-                    const int s1 = (int)((w.s.y >> (g4 * 8u)) & 0xFFu);
-                    c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a1, l1, c[r][m], 4, 0, 0,
-                                                                               s1, 0, 127);
-                }
-#pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    acc[r][m][j].x = fmaf(yd, c[r][m].x, acc[r][m][j].x);
-                    acc[r][m][j].y = fmaf(yd, c[r][m].y, acc[r][m][j].y);
-                    acc[r][m][j].z = fmaf(yd, c[r][m].z, acc[r][m][j].z);
-                    acc[r][m][j].w = fmaf(yd, c[r][m].w, acc[r][m][j].w);
-                }
-            // keep the next column group's operand loads from being hoisted above this one
-            __builtin_amdgcn_sched_barrier(0);
-            if (j == 1 && more) {  // second half of the next tile's staging
-                stage_store(buf ^ 1u, 0);
-                stage_load(sb + 1u, 1);
+                    for (int m = 0; m < 2; m++) {
+                        acc[r][m][j].x = fmaf(yd_prev, c[r][m].x, acc[r][m][j].x);
+                        acc[r][m][j].y = fmaf(yd_prev, c[r][m].y, acc[r][m][j].y);
+                        acc[r][m][j].z = fmaf(yd_prev, c[r][m].z, acc[r][m][j].z);
+                        acc[r][m][j].w = fmaf(yd_prev, c[r][m].w, acc[r][m][j].w);
+                    }
             }
         }
         if (more) {
