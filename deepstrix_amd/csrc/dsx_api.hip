@@ -134,6 +134,11 @@ int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
     const uint32_t per_xcd = (max_wi + 7u) / 8u;
     const uint64_t grid = (uint64_t)8u * per_xcd * p.n_row_tiles;
     if (grid > 0x7FFFFFFFull) return fail(DSX_ERR_INVALID_ARG, "gemm: grid too large");
+    // the kernel addresses weights and activations with 32-bit byte offsets from their bases
+    const uint64_t act_rows = (uint64_t)p.n_tokens * (p.n_used + 1u);
+    if ((uint64_t)p.n_rows * p.n_sb * kSuperBytes > 0xFFFFFFFFull ||
+        act_rows * p.act_row_bytes > 0xFFFFFFFFull)
+        return fail(DSX_ERR_INVALID_ARG, "gemm: a weight matrix or the activation rows exceed 4 GiB");
     hipLaunchKernelGGL((k_mxfp4_gemm<PAIR>), dim3((uint32_t)grid), dim3(kGemmWaves * 64), kGemmLdsBytes,
                        st, p);
     return launched(PAIR ? "gate_up gemm" : "down gemm");

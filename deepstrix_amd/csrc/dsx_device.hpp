@@ -131,6 +131,25 @@ __device__ __forceinline__ void stage_q8k_block(uint8_t *tile, float *yd_slot,
     if (lane == 0) *yd_slot = *(const float *)blk;
 }
 
+// LDS-direct loads: lane l of the wave fetches `size` bytes from its global address and the
+// hardware writes them to LDS at lds_addr + size * l (lds_addr uniform, passed in M0); no
+// vector register holds the data.  They count in vmcnt like any load; the compiler does not
+// see them, so the caller waits (s_waitcnt vmcnt) before the LDS reads that depend on them.
+// `base` must be uniform; `off` is the lane's unsigned byte offset from it.
+__device__ __forceinline__ void lds_dma16(uint32_t lds_addr, const void *base, uint32_t off) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_dma4(uint32_t lds_addr, const void *base, uint32_t off) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+// per-lane 64-bit address form
+__device__ __forceinline__ void lds_dma4_v(uint32_t lds_addr, const void *ptr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off"
+                 :: "s"(lds_addr), "v"(ptr) : "memory");
+}
+
 // Weights of one super-block for the lane's row: its two nibble blocks (halves 0 and 1,
 // block kb of each) and the 8 scale bytes.
 struct WSuper {

@@ -32,7 +32,9 @@ constexpr int kGemmWaves = 4;
 constexpr int kGemmRF = 4;                  // 16-row fragments per wave and row set
 constexpr int kGemmMT = 64;                 // token columns per workgroup
 constexpr int kGemmTileBytes = kGemmMT * 512;  // one super-block of 64 columns in LDS
-constexpr size_t kGemmLdsBytes = 2 * kGemmTileBytes + 2 * kGemmMT * sizeof(float);
+constexpr int kGemmAWaveBytes = 8 * 2048 + 1024;   // a wave's weights of one super-block in LDS
+constexpr int kGemmAOff = 2 * kGemmTileBytes + 2 * kGemmMT * (int)sizeof(float);
+constexpr size_t kGemmLdsBytes = kGemmAOff + kGemmWaves * kGemmAWaveBytes;
 
 struct GemmParams {
     const uint8_t *w0, *w1;        // [n_expert] experts (gate, up), or down in w0 (w1 unused)
@@ -58,10 +60,6 @@ __device__ __forceinline__ uint32_t gemm_dest_row(uint32_t m, uint32_t n_tokens,
     const uint32_t t = m >> 16, slot = m & 0xFFFFu;
     return slot >= n_used ? n_tokens * n_used + t : t * n_used + slot;
 }
-
-struct GemmA {  // the lane's weights of one super-block: row fragments x 2 row sets
-    WSuper f[kGemmRF][2];
-};
 
 template <bool PAIR>
 __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams p) {
@@ -106,7 +104,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
         if (PAIR) s_ew[tid] = (m & 0xFFFFu) >= p.n_used ? 1.0f : p.ew[dest];
     }
 
-    const uint64_t row_stride = (uint64_t)p.n_sb * kSuperBytes;
+    const uint32_t row_stride = p.n_sb * kSuperBytes;
     const uint8_t *wbase[2];
     uint32_t row0[2];
     if (PAIR) {
@@ -118,59 +116,86 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
         row0[0] = rt * 512u;
         row0[1] = rt * 512u + 256u;
     }
-    const uint8_t *wrow[kGemmRF][2];
+    __syncthreads();  // s_src visible
+
+    // ---- data movement: global memory -> LDS without passing through registers ------------
+    // A load whose consecutive lanes read consecutive addresses costs the L1 a quarter of what
+    // the matrix instruction's own operand layout (lane -> row lane % 16) costs, because the L1
+    // looks up one cache line per cycle and a group of four lanes then shares a line.  So both
+    // operands are fetched in memory order by LDS-direct loads (lane l of an instruction writes
+    // LDS bytes [16 l, 16 l + 16) of the instruction's 1 KB destination) and read back from
+    // LDS in operand order.  The 16-byte chunk a lane fetches is XOR-swizzled with its row so
+    // that the later reads, 16 rows at a fixed chunk, spread over all banks.
+    //
+    // A, per wave and super-block: 8 fragments x (16 rows x 128 B of nibbles) + 128 rows x 8 B
+    // of scales, private to the wave (no barrier).  B: the 64 columns' 512 B, shared, double
+    // buffered; wave w fetches columns 16 w .. 16 w + 15.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmAOff + wave * kGemmAWaveBytes);
+    const uint8_t *a_ptr = smem + kGemmAOff + wave * kGemmAWaveBytes;
+    const uint32_t l8 = lane >> 3, c8 = (lane & 7u) ^ l8;
+    // fetch side: lane -> row l8 of the 8-row slab, chunk c8
+    const uint32_t a_fetch = l8 * row_stride + c8 * 16u;
+    uint32_t a_slab[kGemmRF][2];  // first row of fragment (r, m), times the row stride
 #pragma unroll
     for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
         for (int m = 0; m < 2; m++)
-            wrow[r][m] = wbase[m] + (uint64_t)(row0[m] + wave * 64u + r * 16u + n16) * row_stride;
-
-    auto load_a = [&](GemmA &a, uint32_t sb) {
+            a_slab[r][m] = __builtin_amdgcn_readfirstlane((row0[m] + wave * 64u + r * 16u) * row_stride);
+    // scales: lane -> (row set lane / 32, row (lane % 32) / 2, dword lane % 2) of fragment pair r
+    const uint8_t *sc_ptr = wbase[lane >> 5] +
+                            (uint64_t)(row0[lane >> 5] + wave * 64u + ((lane & 31u) >> 1)) * row_stride +
+                            128u + (lane & 1u) * 4u;
+    auto issue_a = [&](uint32_t sb) {
 #pragma unroll
         for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
-            for (int m = 0; m < 2; m++) a.f[r][m] = load_wsuper(wrow[r][m] + (uint64_t)sb * kSuperBytes, g4);
+            for (int m = 0; m < 2; m++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    lds_dma16(a_lds + (uint32_t)((r * 2 + m) * 2048 + i * 1024), wbase[m],
+                              a_slab[r][m] + (uint32_t)i * 8u * row_stride + a_fetch + sb * kSuperBytes);
+#pragma unroll
+        for (int r = 0; r < kGemmRF; r++)
+            lds_dma4_v(a_lds + 16384u + (uint32_t)r * 256u,
+                       sc_ptr + (uint64_t)r * 16u * row_stride + sb * kSuperBytes);
+    };
+    // read side: lane (row n16, block g4) of fragment f: chunk g4 (first half), 4 + g4 (second)
+    const uint32_t sw = ((n16 & 7u) * 8u + (g4 ^ (n16 & 7u))) * 16u;  // within a 1 KB slab
+    const uint32_t a_rd = (n16 >> 3) * 1024u + sw;
+    struct GemmAFrag { uint4 a0, a1; uint2 s; };
+    GemmAFrag a_cur[kGemmRF][2];
+    auto read_a = [&]() {
+#pragma unroll
+        for (int r = 0; r < kGemmRF; r++)
+#pragma unroll
+            for (int m = 0; m < 2; m++) {
+                const uint8_t *f = a_ptr + (r * 2 + m) * 2048;
+                a_cur[r][m].a0 = *(const uint4 *)(f + a_rd);
+                a_cur[r][m].a1 = *(const uint4 *)(f + (a_rd ^ 64u));
+                a_cur[r][m].s = *(const uint2 *)(a_ptr + 16384u + r * 256u + m * 128u + n16 * 8u);
+            }
     };
 
-    GemmA a_cur, a_nxt;
-    load_a(a_cur, 0);
-    __syncthreads();  // s_src visible
+    const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 8192u);
+    uint32_t b_fetch[2];  // column 16 w + 8 ii + l8, chunk c8 of each 128-byte run
+#pragma unroll
+    for (int ii = 0; ii < 2; ii++)
+        b_fetch[ii] = s_src[wave * 16u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
+    const uint32_t yd_fetch = s_src[lane] * p.act_row_bytes + p.n_sb * 512u;
+    const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + 2u * kGemmTileBytes);
+    auto issue_b = [&](uint32_t sb, uint32_t buf) {
+#pragma unroll
+        for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                lds_dma16(b_lds + buf * kGemmTileBytes + (uint32_t)((ii * 4 + k) * 1024), p.act,
+                          b_fetch[ii] + sb * 512u + (uint32_t)k * 128u);
+        if (wave == 0) lds_dma4(yd_lds + buf * (kGemmMT * 4u), p.act, yd_fetch + sb * 4u);
+    };
 
-    // Staging: wave w copies columns 16w .. 16w+15, two per lane; a load instruction of the
-    // wave covers 8 columns x 128 contiguous bytes, the LDS side 128 contiguous bytes per
-    // chunk row and 8 lanes.
-    const uint32_t scol = wave * 16u + (lane & 7u), sch = lane >> 3;
-    const uint8_t *srow0 = p.act + (uint64_t)s_src[scol] * p.act_row_bytes + sch * 16u;
-    const uint8_t *srow1 = p.act + (uint64_t)s_src[scol + 8u] * p.act_row_bytes + sch * 16u;
-    const uint8_t *ydrow = p.act + (uint64_t)s_src[tid & (kGemmMT - 1)] * p.act_row_bytes +
-                           (uint64_t)p.n_sb * 512u;
-    // Two halves (the lane's first, then its second column), each held in four named
-    // registers between its load and its LDS store: an array captured by the lambdas would
-    // land in scratch, and both halves at once cost 16 more registers.
-    uint4 sa0, sa1, sa2, sa3;
-    float st_yd = 0.0f;
-    auto stage_load = [&](uint32_t sb, uint32_t half) {
-        const uint8_t *r0 = (half ? srow1 : srow0) + (uint64_t)sb * 512u;
-        sa0 = *(const uint4 *)(r0);
-        sa1 = *(const uint4 *)(r0 + 128u);
-        sa2 = *(const uint4 *)(r0 + 256u);
-        sa3 = *(const uint4 *)(r0 + 384u);
-        if (half == 0u && tid < (uint32_t)kGemmMT) st_yd = *((const float *)ydrow + sb);
-    };
-    auto stage_store = [&](uint32_t buf, uint32_t half) {
-        uint8_t *d = tiles + buf * kGemmTileBytes + (sch * kGemmMT + scol) * 16u + half * 128u;
-        constexpr uint32_t PS = 8u * kGemmMT * 16u;  // 8 chunk rows
-        *(uint4 *)(d) = sa0;
-        *(uint4 *)(d + PS) = sa1;
-        *(uint4 *)(d + 2u * PS) = sa2;
-        *(uint4 *)(d + 3u * PS) = sa3;
-        if (half == 0u && tid < (uint32_t)kGemmMT) s_yd[buf * kGemmMT + tid] = st_yd;
-    };
-    stage_load(0, 0);
-    stage_store(0, 0);
-    stage_load(0, 1);
-    stage_store(0, 1);
-    __syncthreads();
+    issue_a(0);
+    issue_b(0, 0);
 
     v4f acc[kGemmRF][2][4];
 #pragma unroll
@@ -180,26 +205,31 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
 #pragma unroll
             for (int j = 0; j < 4; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
     const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
     for (uint32_t sb = 0; sb < p.n_sb; sb++) {
         const uint32_t buf = sb & 1u;
         const bool more = sb + 1u < p.n_sb;
+        read_a();
+        // the wave's A region is free again once its reads have returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (more) {
-            stage_load(sb + 1u, 0);
-            load_a(a_nxt, sb + 1u);
+            issue_a(sb + 1u);
+            issue_b(sb + 1u, buf ^ 1u);
         }
         const uint8_t *tile = tiles + buf * kGemmTileBytes;
         // A column group j (16 columns) needs four B pieces: (half 0, high plane), (half 0, low),
-        // (half 1, high), (half 1, low).  Piece p of group j lives in chunk rows 2p and 2p + 1:
-        // chunk row i = ((h * 2 + plane) * 2 + c) * 4 + kb, 64 columns of 16 bytes each.
-        // The pieces are walked in order with the next one already loading while the eight
-        // fragments' instructions of the current one issue; the fold of group j - 1 into the
-        // accumulators (acc += d * c) is interleaved with the first piece of group j, right
-        // before each fragment's temporary is overwritten.
-        constexpr uint32_t CR = 4u * kGemmMT * 16u;  // one (h, plane, c) step
+        // (half 1, high), (half 1, low); piece pc of column c is the 128-byte run pc of its
+        // 512 bytes and sits in slab (c / 8) * 4 + pc.  The pieces are walked in order with the
+        // next one already loading while the eight fragments' instructions of the current one
+        // issue; the fold of group j - 1 into the accumulators (acc += d * c) is interleaved
+        // with the first piece of group j, right before each fragment's temporary is
+        // overwritten.
         auto load_piece = [&](int j, int pc) -> v8i {
-            const uint32_t cb = (g4 * kGemmMT + (uint32_t)j * 16u + n16) * 16u;
-            return b_operand(tile, cb + (2u * pc) * CR, cb + (2u * pc + 1u) * CR);
+            const uint32_t cb = ((uint32_t)(2 * j) + (n16 >> 3)) * 4096u + (uint32_t)pc * 1024u + sw;
+            return b_operand(tile, cb, cb ^ 64u);
         };
         v4f c[kGemmRF][2];
         v8i bq = load_piece(0, 0);
@@ -217,8 +247,8 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                     for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
                         for (int m = 0; m < 2; m++) {
-                            const WSuper &w = a_cur.f[r][m];
-                            const U4A8 &aw = pc < 2 ? w.a0 : w.a1;
+                            const GemmAFrag &w = a_cur[r][m];
+                            const uint4 &aw = pc < 2 ? w.a0 : w.a1;
                             const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
                             const int sc = (int)(((pc < 2 ? w.s.x : w.s.y) >> (g4 * 8u)) & 0xFFu);
                             if (pc == 0) {
@@ -238,10 +268,6 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                     bq = bn;
                 }
                 yd_prev = yd;
-                if (j == 1 && more) {  // second half of the next tile's staging
-                    stage_store(buf ^ 1u, 0);
-                    stage_load(sb + 1u, 1);
-                }
             }
         }
         // fold the last group
@@ -259,14 +285,9 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                     }
             }
         }
-        if (more) {
-            if (cnt <= 16u) {  // the column loop ended before its staging step (j == 1)
-                stage_store(buf ^ 1u, 0);
-                stage_load(sb + 1u, 1);
-            }
-            stage_store(buf ^ 1u, 1);
-            a_cur = a_nxt;
-        }
+        // everything this wave fetched for the next super-block has landed before the others
+        // may read it
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
