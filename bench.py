@@ -108,7 +108,7 @@ def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
     del layer
     return {"tokens_per_s": T / dt, "ms_per_layer": dt * 1e3, "zipf_alpha": alpha,
             "top10pct_share": frac, "max_group": int(cnt.max()), "empty_experts": int((cnt == 0).sum()),
-            "column_tiles_of_64": int(np.ceil(cnt / 64).sum()) + T // 64,
+            "column_tiles_of_128": int(np.ceil(cnt / 128).sum()) + T // 128,
             "useful_flop": flops, "useful_TFLOPs": flops / dt / 1e12,
             "mfma_issued": "v_mfma_scale_f32_16x16x128_f8f6f4, A = FP4 weights, B = FP8 planes of the "
                            "int8 activations (two instructions per product)",

@@ -1,39 +1,44 @@
 // dsx_gemm_kernels.hpp -- MXFP4 expert products for many tokens per expert (prefill): a
 // grouped GEMM on the block-scaled matrix instruction.
 //
-// Work item = (expert, first member), the next up to 64 members of that expert are the
-// token columns.  A workgroup (4 waves, one per SIMD, so that each may use the whole
-// 512-entry register file) multiplies 2 x 256 weight rows with those 64 columns over the
-// whole k range:
+// Work item = (expert, first member), the next up to 128 members of that expert are the
+// token columns.  A workgroup (8 waves, two per SIMD, 256 registers each) multiplies 2 x 256
+// weight rows with those 128 columns over the whole k range:
 //   gate/up (PAIR):  256 rows of gate and the same 256 rows of up; the epilogue applies the
 //                    clamped SwiGLU and the routing weight, quantizes the 256 results of
 //                    every column as one Q8_K block and writes it in the staged format
 //                    that `down` reads -- the f32 `mid` never goes to memory;
 //   down:            512 rows; the epilogue stores f32 partial rows, one per (token, slot).
-// Wave w owns rows [64 w, 64 w + 64) of both row sets and all 64 columns: 4 x 2 x 4 = 32
-// accumulator fragments.  Column groups past the end of a short group are skipped.  Weights go from global memory straight into the A operand (each
-// wave reads only its own rows, so staging them in LDS would add traffic and save none);
-// the 64 columns' activations for one super-block (32 KB of FP8 planes) are staged in LDS,
-// double buffered, and shared by all waves.
+// Wave w owns rows [32 w, 32 w + 32) of both row sets and all 128 columns: 2 x 2 x 8 = 32
+// accumulator fragments.  Column groups past the end of a short group are skipped.
+//
+// The kernel is bound by the bytes that pass through the CU's L1, which serves requests in
+// order: one HBM miss holds back the L2 hits behind it, so every byte moves at about HBM
+// speed (about 19 GB/s per CU) whether or not it hits in L2.  Hence the wide tile (weight
+// bytes per product halve against 64 columns) and loads in memory order (see below).
 //
 // The Q8_K block scale d of the activations differs per (column, super-block), so the
-// matrix pipe cannot carry a sum across super-blocks: each fragment's four instructions of
-// one super-block accumulate into a fresh register quad that is then folded into the
+// matrix pipe cannot carry a sum across super-blocks: each fragment's instructions of one
+// half super-block accumulate into a fresh register quad that is then folded into the
 // accumulator with the column's d (one FMA per value, on the vector ALU while the matrix
 // pipe runs the next fragment).
 #pragma once
+
+#include <type_traits>
 
 #include "dsx_device.hpp"
 #include "dsx_quant.hpp"
 
 namespace dsx {
 
-constexpr int kGemmWaves = 4;
-constexpr int kGemmRF = 4;                  // 16-row fragments per wave and row set
-constexpr int kGemmMT = 64;                 // token columns per workgroup
-constexpr int kGemmTileBytes = kGemmMT * 512;  // one super-block of 64 columns in LDS
-constexpr int kGemmAWaveBytes = 8 * 2048 + 1024;   // a wave's weights of one super-block in LDS
-constexpr int kGemmAOff = 2 * kGemmTileBytes + 2 * kGemmMT * (int)sizeof(float);
+constexpr int kGemmWaves = 8;
+constexpr int kGemmRF = 2;                  // 16-row fragments per wave and row set
+constexpr int kGemmMT = 128;                // token columns per workgroup
+constexpr int kGemmCG = kGemmMT / 16;       // column groups
+constexpr int kGemmHalfBytes = kGemmMT * 256;  // half a super-block of all columns in LDS
+constexpr int kGemmAWaveBytes = 2 * kGemmRF * 2048 + 2 * 256;  // a wave's weights of one super-block
+constexpr int kGemmYdOff = 2 * kGemmHalfBytes;
+constexpr int kGemmAOff = kGemmYdOff + 2 * kGemmMT * (int)sizeof(float);
 constexpr size_t kGemmLdsBytes = kGemmAOff + kGemmWaves * kGemmAWaveBytes;
 
 struct GemmParams {
@@ -71,15 +76,15 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     __shared__ float s_iscale[kGemmMT];
 
     uint8_t *tiles = smem;
-    float *s_yd = (float *)(smem + 2 * kGemmTileBytes);
+    float *s_yd = (float *)(smem + kGemmYdOff);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t g4 = lane >> 4, n16 = lane & 15u;
 
     // Workgroups are dealt to the 8 XCDs round-robin by id, and each XCD has its own L2.  An
-    // XCD gets a contiguous range of work items; its 32 concurrent workgroups are then four
-    // consecutive items (usually column tiles of the same expert: they stream the same weights
-    // in step) times the eight row tiles of each (they stream the same activations).
+    // XCD gets a contiguous range of work items; its 32 concurrent workgroups are then a few
+    // consecutive items (often column tiles of the same expert: they stream the same weights
+    // in step) times the row tiles of each (they stream the same activations).
     const uint32_t xcd = blockIdx.x & 7u, seq = blockIdx.x >> 3;
     const uint32_t n_items = (uint32_t)*p.n_work_items;   // the grid is only an upper bound
     const uint32_t items_per_xcd = (n_items + 7u) / 8u;
@@ -127,9 +132,12 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     // LDS in operand order.  The 16-byte chunk a lane fetches is XOR-swizzled with its row so
     // that the later reads, 16 rows at a fixed chunk, spread over all banks.
     //
-    // A, per wave and super-block: 8 fragments x (16 rows x 128 B of nibbles) + 128 rows x 8 B
-    // of scales, private to the wave (no barrier).  B: the 64 columns' 512 B, shared, double
-    // buffered; wave w fetches columns 16 w .. 16 w + 15.
+    // A, per wave and super-block: 4 fragments x (16 rows x 128 B of nibbles) + 64 rows x 8 B
+    // of scales, private to the wave (no barrier).  B: the 128 columns' 256 B of half a
+    // super-block, shared, double buffered; wave w fetches columns 16 w .. 16 w + 15.
+    constexpr uint32_t kRowsPerWave = 16u * kGemmRF;
+    static_assert(kGemmRF == 2, "one scale instruction covers the 32 rows of a wave's row set");
+    constexpr uint32_t kScaleOff = 2u * kGemmRF * 2048u;
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmAOff + wave * kGemmAWaveBytes);
     const uint8_t *a_ptr = smem + kGemmAOff + wave * kGemmAWaveBytes;
@@ -141,11 +149,9 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
         for (int m = 0; m < 2; m++)
-            a_slab[r][m] = __builtin_amdgcn_readfirstlane((row0[m] + wave * 64u + r * 16u) * row_stride);
-    // scales: lane -> (row set lane / 32, row (lane % 32) / 2, dword lane % 2) of fragment pair r
-    const uint8_t *sc_ptr = wbase[lane >> 5] +
-                            (uint64_t)(row0[lane >> 5] + wave * 64u + ((lane & 31u) >> 1)) * row_stride +
-                            128u + (lane & 1u) * 4u;
+            a_slab[r][m] = __builtin_amdgcn_readfirstlane((row0[m] + wave * kRowsPerWave + r * 16u) * row_stride);
+    // scales: one instruction per row set, lane -> (row lane / 2 of the wave's 32, dword lane % 2)
+    const uint32_t sc_fetch = (lane >> 1) * row_stride + 128u + (lane & 1u) * 4u;
     auto issue_a = [&](uint32_t sb) {
 #pragma unroll
         for (int r = 0; r < kGemmRF; r++)
@@ -156,14 +162,16 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                     lds_dma16(a_lds + (uint32_t)((r * 2 + m) * 2048 + i * 1024), wbase[m],
                               a_slab[r][m] + (uint32_t)i * 8u * row_stride + a_fetch + sb * kSuperBytes);
 #pragma unroll
-        for (int r = 0; r < kGemmRF; r++)
-            lds_dma4_v(a_lds + 16384u + (uint32_t)r * 256u,
-                       sc_ptr + (uint64_t)r * 16u * row_stride + sb * kSuperBytes);
+        for (int m = 0; m < 2; m++)
+            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m],
+                     a_slab[0][m] + sc_fetch + sb * kSuperBytes);
     };
+    constexpr int kALoads = 4 * kGemmRF + 2;  // per wave and super-block
     // read side: lane (row n16, block g4) of fragment f: chunk g4 (first half), 4 + g4 (second)
     const uint32_t sw = ((n16 & 7u) * 8u + (g4 ^ (n16 & 7u))) * 16u;  // within a 1 KB slab
     const uint32_t a_rd = (n16 >> 3) * 1024u + sw;
-    struct GemmAFrag { uint4 a0, a1; uint2 s; };
+    // sc: the lane's two scale bytes (block g4 of the first and of the second half), bytes 0 and 1
+    struct GemmAFrag { uint4 a0, a1; uint32_t sc; };
     GemmAFrag a_cur[kGemmRF][2];
     auto read_a = [&]() {
 #pragma unroll
@@ -173,96 +181,91 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                 const uint8_t *f = a_ptr + (r * 2 + m) * 2048;
                 a_cur[r][m].a0 = *(const uint4 *)(f + a_rd);
                 a_cur[r][m].a1 = *(const uint4 *)(f + (a_rd ^ 64u));
-                a_cur[r][m].s = *(const uint2 *)(a_ptr + 16384u + r * 256u + m * 128u + n16 * 8u);
+                const uint2 sv = *(const uint2 *)(a_ptr + kScaleOff + m * 256u + r * 128u + n16 * 8u);
+                a_cur[r][m].sc = ((sv.x >> (g4 * 8u)) & 0xFFu) | (((sv.y >> (g4 * 8u)) & 0xFFu) << 8);
             }
     };
 
-    const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 8192u);
+    // B half h of super-block sb: bytes [256 h, 256 h + 256) of each column's 512; its 128-byte
+    // run q (piece 2 h + q) of the 8 columns 8 g .. 8 g + 7 is slab 2 g + q of the half buffer.
+    const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 4096u);
     uint32_t b_fetch[2];  // column 16 w + 8 ii + l8, chunk c8 of each 128-byte run
 #pragma unroll
     for (int ii = 0; ii < 2; ii++)
         b_fetch[ii] = s_src[wave * 16u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
-    const uint32_t yd_fetch = s_src[lane] * p.act_row_bytes + p.n_sb * 512u;
-    const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + 2u * kGemmTileBytes);
-    auto issue_b = [&](uint32_t sb, uint32_t buf) {
+    const uint32_t yd_fetch = s_src[tid & (kGemmMT - 1)] * p.act_row_bytes + p.n_sb * 512u;
+    const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 256u);
+    auto issue_b = [&](uint32_t sb, uint32_t h) {  // into half buffer h
 #pragma unroll
         for (int ii = 0; ii < 2; ii++)
 #pragma unroll
-            for (int k = 0; k < 4; k++)
-                lds_dma16(b_lds + buf * kGemmTileBytes + (uint32_t)((ii * 4 + k) * 1024), p.act,
-                          b_fetch[ii] + sb * 512u + (uint32_t)k * 128u);
-        if (wave == 0) lds_dma4(yd_lds + buf * (kGemmMT * 4u), p.act, yd_fetch + sb * 4u);
+            for (int q = 0; q < 2; q++)
+                lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)((ii * 2 + q) * 1024), p.act,
+                          b_fetch[ii] + sb * 512u + h * 256u + (uint32_t)q * 128u);
+    };
+    auto issue_yd = [&](uint32_t sb) {  // waves 0 and 1: 64 columns each
+        if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * (kGemmMT * 4u), p.act, yd_fetch + sb * 4u);
     };
 
-    issue_a(0);
     issue_b(0, 0);
+    issue_yd(0);
+    issue_a(0);
 
-    v4f acc[kGemmRF][2][4];
+    v4f acc[kGemmRF][2][kGemmCG];
 #pragma unroll
     for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
         for (int m = 0; m < 2; m++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < kGemmCG; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
-    for (uint32_t sb = 0; sb < p.n_sb; sb++) {
-        const uint32_t buf = sb & 1u;
-        const bool more = sb + 1u < p.n_sb;
-        read_a();
-        // the wave's A region is free again once its reads have returned
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (more) {
-            issue_a(sb + 1u);
-            issue_b(sb + 1u, buf ^ 1u);
-        }
-        const uint8_t *tile = tiles + buf * kGemmTileBytes;
-        // A column group j (16 columns) needs four B pieces: (half 0, high plane), (half 0, low),
-        // (half 1, high), (half 1, low); piece pc of column c is the 128-byte run pc of its
-        // 512 bytes and sits in slab (c / 8) * 4 + pc.  The pieces are walked in order with the
-        // next one already loading while the eight fragments' instructions of the current one
-        // issue; the fold of group j - 1 into the accumulators (acc += d * c) is interleaved
-        // with the first piece of group j, right before each fragment's temporary is
-        // overwritten.
-        auto load_piece = [&](int j, int pc) -> v8i {
-            const uint32_t cb = ((uint32_t)(2 * j) + (n16 >> 3)) * 4096u + (uint32_t)pc * 1024u + sw;
-            return b_operand(tile, cb, cb ^ 64u);
+    // One half super-block: for every column group, the two pieces (high and low plane) against
+    // the wave's four fragments, then the fold acc += d * c -- interleaved with the first
+    // piece of the next group, right before each fragment's temporary is overwritten.
+    auto compute_half = [&](auto hc, const uint32_t sb) {
+        constexpr int h = decltype(hc)::value;
+        const uint8_t *half = tiles + h * kGemmHalfBytes;
+        const float *yds = s_yd + (sb & 1u) * kGemmMT;
+        auto load_piece = [&](int j, int q) -> v8i {
+            const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 2u + (uint32_t)q) * 1024u + sw;
+            return b_operand(half, cb, cb ^ 64u);
         };
         v4f c[kGemmRF][2];
         v8i bq = load_piece(0, 0);
         float yd_prev = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kGemmCG; j++) {
             if ((uint32_t)j < nj) {  // uniform
-                const float yd = s_yd[buf * kGemmMT + j * 16u + n16];
+                const float yd = yds[j * 16u + n16];
 #pragma unroll
-                for (int pc = 0; pc < 4; pc++) {
+                for (int q = 0; q < 2; q++) {
                     v8i bn = bq;
-                    if (pc < 3) bn = load_piece(j, pc + 1);
-                    else if (j < 3 && (uint32_t)(j + 1) < nj) bn = load_piece(j + 1, 0);
+                    if (q == 0) bn = load_piece(j, 1);
+                    else if (j + 1 < kGemmCG && (uint32_t)(j + 1) < nj) bn = load_piece(j + 1, 0);
 #pragma unroll
                     for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
                         for (int m = 0; m < 2; m++) {
                             const GemmAFrag &w = a_cur[r][m];
-                            const uint4 &aw = pc < 2 ? w.a0 : w.a1;
+                            const uint4 &aw = h == 0 ? w.a0 : w.a1;
                             const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
-                            const int sc = (int)(((pc < 2 ? w.s.x : w.s.y) >> (g4 * 8u)) & 0xFFu);
-                            if (pc == 0) {
+                            if (q == 0) {
                                 if (j > 0) {
-                                    acc[r][m][j > 0 ? j - 1 : 0].x = fmaf(yd_prev, c[r][m].x, acc[r][m][j > 0 ? j - 1 : 0].x);
-                                    acc[r][m][j > 0 ? j - 1 : 0].y = fmaf(yd_prev, c[r][m].y, acc[r][m][j > 0 ? j - 1 : 0].y);
-                                    acc[r][m][j > 0 ? j - 1 : 0].z = fmaf(yd_prev, c[r][m].z, acc[r][m][j > 0 ? j - 1 : 0].z);
-                                    acc[r][m][j > 0 ? j - 1 : 0].w = fmaf(yd_prev, c[r][m].w, acc[r][m][j > 0 ? j - 1 : 0].w);
+                                    v4f &a = acc[r][m][j > 0 ? j - 1 : 0];
+                                    a.x = fmaf(yd_prev, c[r][m].x, a.x);
+                                    a.y = fmaf(yd_prev, c[r][m].y, a.y);
+                                    a.z = fmaf(yd_prev, c[r][m].z, a.z);
+                                    a.w = fmaf(yd_prev, c[r][m].w, a.w);
                                 }
                                 c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                                    av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 0, 0, sc, 0, 131);
+                                    av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 0, h, (int)w.sc, 0, 131);
                             } else {
                                 c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                                    av, bq, c[r][m], 4, 0, 0, sc, 0, (pc & 1) ? 127 : 131);
+                                    av, bq, c[r][m], 4, 0, h, (int)w.sc, 0, 127);
                             }
                         }
                     bq = bn;
@@ -272,19 +275,39 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
         }
         // fold the last group
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kGemmCG; j++) {
             if ((uint32_t)j + 1u == nj) {
 #pragma unroll
                 for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
                     for (int m = 0; m < 2; m++) {
-                        acc[r][m][j].x = fmaf(yd_prev, c[r][m].x, acc[r][m][j].x);
-                        acc[r][m][j].y = fmaf(yd_prev, c[r][m].y, acc[r][m][j].y);
-                        acc[r][m][j].z = fmaf(yd_prev, c[r][m].z, acc[r][m][j].z);
-                        acc[r][m][j].w = fmaf(yd_prev, c[r][m].w, acc[r][m][j].w);
+                        v4f &a = acc[r][m][j];
+                        a.x = fmaf(yd_prev, c[r][m].x, a.x);
+                        a.y = fmaf(yd_prev, c[r][m].y, a.y);
+                        a.z = fmaf(yd_prev, c[r][m].z, a.z);
+                        a.w = fmaf(yd_prev, c[r][m].w, a.w);
                     }
             }
         }
+    };
+
+    for (uint32_t sb = 0; sb < p.n_sb; sb++) {
+        const bool more = sb + 1u < p.n_sb;
+        read_a();
+        // the wave's A region is free again once its reads have returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        issue_b(sb, 1);
+        if (more) issue_a(sb + 1u);
+        compute_half(std::integral_constant<int, 0>{}, sb);
+        // the second half of B has landed (the younger weight loads may still be on their way)
+        if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kALoads) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (more) {
+            issue_b(sb + 1u, 0);
+            issue_yd(sb + 1u);
+        }
+        compute_half(std::integral_constant<int, 1>{}, sb);
         // everything this wave fetched for the next super-block has landed before the others
         // may read it
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -292,10 +315,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     }
 
     // ---- epilogue ---------------------------------------------------------------------
-    // The lane holds, for each of its 4 columns j*16 + n16, rows 64w + 16r + 4*g4 + q.
+    // The lane holds, for each of its 8 columns j*16 + n16, rows 32w + 16r + 4*g4 + q.
     if (!PAIR) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kGemmCG; j++) {
             const uint32_t col = j * 16u + n16;
             if (col >= cnt) continue;
             float *dst = p.partials + (uint64_t)s_dest[col] * p.n_rows;
@@ -304,7 +327,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
 #pragma unroll
                 for (int m = 0; m < 2; m++) {
                     const v4f v = acc[r][m][j];
-                    *(float4 *)(dst + row0[m] + wave * 64u + r * 16u + g4 * 4u) =
+                    *(float4 *)(dst + row0[m] + wave * kRowsPerWave + r * 16u + g4 * 4u) =
                         make_float4(v.x, v.y, v.z, v.w);
                 }
         }
@@ -315,7 +338,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     // rows of this tile per column (crates/v4flash-kernels/kernels/q8_k_quantize.hip:23-90:
     // the element of largest |x|, the first one on ties, sets iscale = -127 / x).
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < kGemmCG; j++) {
         const float ew = s_ew[j * 16u + n16];
         uint64_t best = 0;
 #pragma unroll
@@ -329,7 +352,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const float v = q == 0 ? gv.x : q == 1 ? gv.y : q == 2 ? gv.z : gv.w;
-                const uint32_t idx = wave * 64u + r * 16u + g4 * 4u + q;
+                const uint32_t idx = wave * kRowsPerWave + r * 16u + g4 * 4u + q;
                 const uint32_t bits = __float_as_uint(v);
                 const uint64_t key = ((uint64_t)(bits & 0x7FFFFFFFu) << 32) | ((255u - idx) << 1) | (bits >> 31);
                 best = key > best ? key : best;
@@ -344,10 +367,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     }
     if (p.mid != nullptr) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kGemmCG; j++) {
             const uint32_t col = j * 16u + n16;
             if (col >= cnt) continue;
-            float *dst = p.mid + (uint64_t)s_dest[col] * p.n_rows + rt * 256u + wave * 64u + g4 * 4u;
+            float *dst = p.mid + (uint64_t)s_dest[col] * p.n_rows + rt * 256u + wave * kRowsPerWave + g4 * 4u;
 #pragma unroll
             for (int r = 0; r < kGemmRF; r++) {
                 const v4f v = acc[r][0][j];
@@ -375,11 +398,11 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     }
     __syncthreads();
     // Rows 16r + 4*g4 + q of fragments r = 2*rho, 2*rho + 1 are the nibble positions
-    // 8*g4 .. 8*g4+7 of 32-element block 2*wave + rho: 8 consecutive bytes of each plane of
+    // 8*g4 .. 8*g4+7 of 32-element block (kGemmRF / 2) * wave + rho: 8 consecutive bytes of each plane of
     // the staged tile (byte 2*(q & 1) + (r & 1) of dword q / 2).
     const uint32_t plane_step = tile_off<1>(0, 1, 0, 0, 0);
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < kGemmCG; j++) {
         const uint32_t col = j * 16u + n16;
         const float iscale = s_iscale[col];
 #pragma unroll
@@ -402,7 +425,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                 }
             }
             if (col >= cnt) continue;
-            const uint32_t b32 = wave * 2u + rho;
+            const uint32_t b32 = wave * (kGemmRF / 2) + rho;
             const uint32_t hh = b32 >> 2, bb = b32 & 3u;
             const uint32_t toff = tile_off<1>(hh, 0, bb >> 1, 2u * (bb & 1u) + (g4 >> 1), 0) + (g4 & 1u) * 8u;
             uint8_t *dst = p.midq + (uint64_t)s_dest[col] * p.out_row_bytes + (uint64_t)rt * 512u + toff;
