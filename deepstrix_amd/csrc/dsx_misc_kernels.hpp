@@ -589,6 +589,27 @@ __device__ __forceinline__ float block_sum_256(float v, float *red, uint32_t tid
     return red[0] + red[1] + red[2] + red[3];
 }
 
+// Sums of N values over the 256 threads of a workgroup in one pass; every thread gets them.
+// `red` holds 4 * N floats.
+template <int N>
+__device__ __forceinline__ void block_sum_256_multi(float (&v)[N], float *red, uint32_t tid) {
+#pragma unroll
+    for (int k = 0; k < N; k++) v[k] = wave_sum_f32(v[k]);
+    __syncthreads();  // `red` may still be read from a previous call
+    if ((tid & 63u) == 0u) {
+#pragma unroll
+        for (int k = 0; k < N; k++) red[(tid >> 6) * N + k] = v[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < N; k++) v[k] = (red[k] + red[N + k]) + (red[2 * N + k] + red[3 * N + k]);
+}
+
+// One workgroup per expert, up to kRlTokens tokens per pass.  With NORM the row is normalized
+// on the fly: logit = (sum_i w[i] * (x[i] * norm_w[i])) / rms(x) -- the sum of squares and the
+// dot product are accumulated in the same sweep and reduced together, so the kernel has one
+// round of loads on its critical path; the workgroups whose index is a token id then write
+// that token's normalized row.
 template <bool NORM>
 __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logits,
                                                        float *__restrict__ xn,
@@ -597,7 +618,7 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
                                                        const float *__restrict__ norm_w, float eps,
                                                        uint32_t n_expert, uint32_t hidden,
                                                        uint32_t n_tokens) {
-    __shared__ float s_red[4];
+    __shared__ float s_red[4 * 2 * kRlTokens];
     const uint32_t tid = threadIdx.x;
     const uint32_t e = blockIdx.x;
     const float *wr = w + (uint64_t)e * hidden;
@@ -605,26 +626,14 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
     const uint32_t n4 = (hidden % 4u == 0u) ? hidden / 4u : 0u;
     for (uint32_t t0 = 0; t0 < n_tokens; t0 += kRlTokens) {
         const uint32_t nt = min((uint32_t)kRlTokens, n_tokens - t0);
-        float scale[kRlTokens];
+        float acc[kRlTokens];
+        double sq[kRlTokens];  // sum of squares with f64 partial sums, like k_rms_norm
 #pragma unroll
         for (int j = 0; j < kRlTokens; j++) {
-            scale[j] = 1.0f;
-            if (NORM && (uint32_t)j < nt) {
-                // mean of squares with f64 partial sums, like k_rms_norm
-                const float *xr = x + (uint64_t)(t0 + j) * hidden;
-                double partial = 0.0;
-                for (uint32_t i = tid; i < n4; i += 256u) {
-                    const float4 v = *(const float4 *)(xr + 4u * i);
-                    partial += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
-                }
-                for (uint32_t i = 4u * n4 + tid; i < hidden; i += 256u) partial += (double)xr[i] * xr[i];
-                const float ss = block_sum_256((float)partial, s_red, tid);
-                scale[j] = 1.0f / sqrtf(ss / (float)hidden + eps);
-            }
+            acc[j] = 0.0f;
+            sq[j] = 0.0;
         }
-        float acc[kRlTokens];
-#pragma unroll
-        for (int j = 0; j < kRlTokens; j++) acc[j] = 0.0f;
+#pragma unroll 4
         for (uint32_t i = tid; i < n4; i += 256u) {
             const float4 wv = *(const float4 *)(wr + 4u * i);
             float4 nw = {1.f, 1.f, 1.f, 1.f};
@@ -634,12 +643,12 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
                 if ((uint32_t)j < nt) {
                     float4 xv = *(const float4 *)(x + (uint64_t)(t0 + j) * hidden + 4u * i);
                     if (NORM) {
-                        xv.x = xv.x * scale[j] * nw.x;
-                        xv.y = xv.y * scale[j] * nw.y;
-                        xv.z = xv.z * scale[j] * nw.z;
-                        xv.w = xv.w * scale[j] * nw.w;
-                        if (e == t0 + j)
-                            *(float4 *)(xn + (uint64_t)(t0 + j) * hidden + 4u * i) = xv;
+                        sq[j] += (double)xv.x * xv.x + (double)xv.y * xv.y + (double)xv.z * xv.z +
+                                 (double)xv.w * xv.w;
+                        xv.x *= nw.x;
+                        xv.y *= nw.y;
+                        xv.z *= nw.z;
+                        xv.w *= nw.w;
                     }
                     acc[j] = fmaf(wv.x, xv.x, acc[j]);
                     acc[j] = fmaf(wv.y, xv.y, acc[j]);
@@ -655,18 +664,40 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
                 if ((uint32_t)j < nt) {
                     float xv = x[(uint64_t)(t0 + j) * hidden + i];
                     if (NORM) {
-                        xv = xv * scale[j] * norm_w[i];
-                        if (e == t0 + j) xn[(uint64_t)(t0 + j) * hidden + i] = xv;
+                        sq[j] += (double)xv * xv;
+                        xv *= norm_w[i];
                     }
                     acc[j] = fmaf(wv, xv, acc[j]);
                 }
             }
         }
+        float red[2 * kRlTokens];
+#pragma unroll
+        for (int j = 0; j < kRlTokens; j++) {
+            red[j] = acc[j];
+            red[kRlTokens + j] = (float)sq[j];
+        }
+        block_sum_256_multi<2 * kRlTokens>(red, s_red, tid);
 #pragma unroll
         for (int j = 0; j < kRlTokens; j++) {
             if ((uint32_t)j < nt) {
-                const float v = block_sum_256(acc[j], s_red, tid);
-                if (tid == 0) logits[(uint64_t)(t0 + j) * n_expert + e] = v;
+                const float scale = NORM ? 1.0f / sqrtf(red[kRlTokens + j] / (float)hidden + eps) : 1.0f;
+                if (tid == 0) logits[(uint64_t)(t0 + j) * n_expert + e] = red[j] * scale;
+                if (NORM && e == t0 + (uint32_t)j) {
+                    const float *xr = x + (uint64_t)e * hidden;
+                    float *xo = xn + (uint64_t)e * hidden;
+                    for (uint32_t i = tid; i < n4; i += 256u) {
+                        float4 xv = *(const float4 *)(xr + 4u * i);
+                        const float4 nw = *(const float4 *)(norm_w + 4u * i);
+                        xv.x = xv.x * scale * nw.x;
+                        xv.y = xv.y * scale * nw.y;
+                        xv.z = xv.z * scale * nw.z;
+                        xv.w = xv.w * scale * nw.w;
+                        *(float4 *)(xo + 4u * i) = xv;
+                    }
+                    for (uint32_t i = 4u * n4 + tid; i < hidden; i += 256u)
+                        xo[i] = xr[i] * scale * norm_w[i];
+                }
             }
         }
     }
