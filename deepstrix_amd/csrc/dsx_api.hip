@@ -317,10 +317,15 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     p.residual = residual;
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.n_slots = n_slots;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
+    // two workgroups of 8 waves per CU, all resident at once and of equal size where the row
+    // count allows (7168 rows on 256 CUs: 512 workgroups of 14 rows)
+    const uint32_t even = (n_rows + 2u * g_num_cu - 1u) / (2u * g_num_cu);
+    p.rows_per_wg = std::min(16u, std::max(8u, even));
+    const uint32_t gx = (n_rows + p.rows_per_wg - 1u) / p.rows_per_wg;
     if (staged)
-        hipLaunchKernelGGL(k_mxfp4_down_decode<true>, dim3(n_rows / 16, n_tokens), dim3(kDownWaves * 64), lds, st, p);
+        hipLaunchKernelGGL(k_mxfp4_down_decode<true>, dim3(gx, n_tokens), dim3(kDownWaves * 64), lds, st, p);
     else
-        hipLaunchKernelGGL(k_mxfp4_down_decode<false>, dim3(n_rows / 16, n_tokens), dim3(kDownWaves * 64), lds, st, p);
+        hipLaunchKernelGGL(k_mxfp4_down_decode<false>, dim3(gx, n_tokens), dim3(kDownWaves * 64), lds, st, p);
     return launched("moe_down_batched");
 }
 

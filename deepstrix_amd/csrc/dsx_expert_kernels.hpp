@@ -317,6 +317,7 @@ struct DownDecodeParams {
     const float *residual;    // [n_tokens, n_rows] added to the result (may alias out), or null
     uint64_t dbpe;
     uint32_t xq_slot_stride, n_used, n_slots, n_rows, n_blocks_in;
+    uint32_t rows_per_wg;     // output rows of one workgroup, at most 16: the grid is sized to fill the CUs evenly
 };
 
 // LDS: [n_slots * n_blocks_in] tiles of 512 bytes | yd[n_slots * n_blocks_in]
@@ -332,8 +333,11 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     float *s_yd = (float *)(smem + (size_t)units * 512u);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t row0 = blockIdx.x * 16u;
+    const uint32_t row0 = blockIdx.x * p.rows_per_wg;
     const uint32_t r = lane & 15u, kb = lane >> 4;
+    // rows of the 16-row fragment past the workgroup's share (or the matrix) load nothing
+    const uint32_t n_live = min(p.rows_per_wg, p.n_rows - row0);
+    const bool live = r < n_live;
     const uint64_t row_off = (uint64_t)(row0 + r) * nb * kSuperBytes;
     // blockIdx.y = token: its picks, its n_slots activation rows, its output row
     const int32_t *selected = p.selected + (uint64_t)blockIdx.y * p.n_used;
@@ -351,11 +355,11 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     // five (slot, super-block) units of weights in flight per wave
     uint32_t un = wave;
     WSuper w0 = {}, w1 = {}, w2 = {}, w3 = {}, w4 = {};
-    if (un < units) w0 = load_wsuper(unit_ptr(un), kb);
-    if (un + kDownWaves < units) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
-    if (un + 2 * kDownWaves < units) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
-    if (un + 3 * kDownWaves < units) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
-    if (un + 4 * kDownWaves < units) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
+    if (un < units && live) w0 = load_wsuper(unit_ptr(un), kb);
+    if (un + kDownWaves < units && live) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
+    if (un + 2 * kDownWaves < units && live) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
+    if (un + 3 * kDownWaves < units && live) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
+    if (un + 4 * kDownWaves < units && live) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
 
     if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? selected[tid] : 0;
     if (STAGED) {
@@ -379,7 +383,7 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     };
 #define DSX_DOWN_STEP(W)                                                                     \
     compute(un, W);                                                                          \
-    if (un + 5 * kDownWaves < units) W = load_wsuper(unit_ptr(un + 5 * kDownWaves), kb);     \
+    if (un + 5 * kDownWaves < units && live) W = load_wsuper(unit_ptr(un + 5 * kDownWaves), kb); \
     un += kDownWaves;                                                                        \
     if (un >= units) break;
     while (un < units) {
@@ -396,7 +400,7 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     s_red[wave][2][lane] = acc.z;
     s_red[wave][3][lane] = acc.w;
     __syncthreads();
-    if (tid < 16u) {
+    if (tid < n_live) {
         const uint32_t l = (tid >> 2) * 16u, i = tid & 3u;
         float s = 0.0f;
 #pragma unroll
