@@ -195,7 +195,11 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
         b_fetch[ii] = s_src[wave * 16u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
     const uint32_t yd_fetch = s_src[tid & (kGemmMT - 1)] * p.act_row_bytes + p.n_sb * 512u;
     const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 256u);
+    // a wave whose 16 columns lie past the end of a short group fetches nothing (nobody reads
+    // them: the column loop stops at the last group that holds a real column)
+    const bool b_live = wave * 16u < cnt;
     auto issue_b = [&](uint32_t sb, uint32_t h) {  // into half buffer h
+        if (!b_live) return;
 #pragma unroll
         for (int ii = 0; ii < 2; ii++)
 #pragma unroll
