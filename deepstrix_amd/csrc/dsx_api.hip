@@ -365,7 +365,9 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
                                  const int32_t *expert_members, const int32_t *work_items,
                                  const int32_t *n_work_items, uint32_t max_work_items,
                                  uint64_t gbpe, uint64_t ubpe, uint32_t n_used, uint32_t chunk,
-                                 float clamp, uint32_t n_rows, uint32_t n_blocks, bool staged) {
+                                 float clamp, uint32_t n_rows, uint32_t n_blocks, bool staged,
+                                 const uint8_t *sh_gate = nullptr, const uint8_t *sh_up = nullptr,
+                                 float sh_clamp = 0.0f, uint32_t n_expert = 0, uint32_t n_tokens = 0) {
     if (max_work_items == 0) return DSX_OK;
     if (!mid || !gate || !up || !xq || !ew || !group_count || !group_offset || !expert_members ||
         !work_items || !n_work_items)
@@ -398,6 +400,7 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used; p.chunk = chunk; p.clamp = clamp;
     p.n_rows = n_rows; p.n_blocks = n_blocks;
     p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
+    p.sh_gate = sh_gate; p.sh_up = sh_up; p.sh_clamp = sh_clamp; p.n_expert = n_expert; p.n_tokens = n_tokens;
     hipStream_t st = S(stream);
     switch (nt) {
         case 1: launch_gate_up_be<1>(st, p, max_work_items, lds, staged); break;
@@ -426,7 +429,8 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
                            const int32_t *work_items, const int32_t *n_work_items,
                            uint32_t max_work_items, uint64_t dbpe, uint32_t xq_slot_stride,
                            uint32_t n_used, uint32_t chunk, uint32_t n_rows, uint32_t n_blocks_in,
-                           bool staged) {
+                           bool staged, const uint8_t *sh_down = nullptr, uint32_t n_expert = 0,
+                           uint32_t n_tokens = 0) {
     if (max_work_items == 0) return DSX_OK;
     if (!partials || !down || !xq || !group_count || !group_offset || !expert_members ||
         !work_items || !n_work_items)
@@ -460,6 +464,7 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
     p.work_items = work_items; p.n_work_items = n_work_items;
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
+    p.sh_down = sh_down; p.n_expert = n_expert; p.n_tokens = n_tokens;
     hipStream_t st = S(stream);
     switch (nt) {
         case 1: launch_down_be<1>(st, p, max_work_items, lds, staged); break;

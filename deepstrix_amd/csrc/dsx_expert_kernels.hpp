@@ -109,6 +109,9 @@ struct GateUpParams {
     uint32_t n_used, chunk;
     float clamp, sh_clamp;
     uint32_t n_rows, n_blocks, xq_row_bytes, midp_row_bytes;
+    // by-expert with the extra expert (index n_expert, slot n_used; its rows follow the
+    // n_tokens * n_used routed ones): sh_gate / sh_up / sh_clamp above, and
+    uint32_t n_expert, n_tokens;
 };
 
 // LDS: [n_blocks] tiles of 512 * NT bytes | yd[n_blocks * NT] floats
@@ -140,15 +143,17 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         cnt = min(p.chunk, total - start);
         if (cnt > (uint32_t)NT) cnt = NT;
         const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+        const bool extra = p.sh_gate != nullptr && e >= p.n_expert;
         if (tid < cnt) {
             const uint32_t m = (uint32_t)p.members[mbase + tid];
             const uint32_t t = m >> 16, slot = m & 0xFFFFu;
             s_tok[tid] = t;
-            s_dest[tid] = (int)(t * p.n_used + slot);
-            s_ew[tid] = p.ew[t * p.n_used + slot];
+            s_dest[tid] = (int)(slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot);
+            s_ew[tid] = slot >= p.n_used ? 1.0f : p.ew[t * p.n_used + slot];
         }
-        gate_e = p.gate + (uint64_t)e * p.gbpe;
-        up_e = p.up + (uint64_t)e * p.ubpe;
+        gate_e = extra ? p.sh_gate : p.gate + (uint64_t)e * p.gbpe;
+        up_e = extra ? p.sh_up : p.up + (uint64_t)e * p.ubpe;
+        if (extra) clamp = p.sh_clamp;
     } else {
         // decode: item = token * n_slots + slot; slot n_used is the extra (shared) expert
         cnt = 1;
@@ -422,6 +427,8 @@ struct DownByExpertParams {
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
     uint64_t dbpe;
     uint32_t xq_slot_stride, n_used, chunk, n_rows, n_blocks_in;
+    const uint8_t *sh_down;  // the extra expert (index n_expert, slot n_used), or null
+    uint32_t n_expert, n_tokens;
 };
 
 // LDS: [n_blocks_in] tiles of 512 * NT bytes | yd[n_blocks_in * NT]
@@ -445,13 +452,16 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     uint32_t cnt = min(p.chunk, (uint32_t)p.group_count[e] - start);
     if (cnt > (uint32_t)NT) cnt = NT;
     const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+    const bool extra = p.sh_down != nullptr && e >= p.n_expert;
     if (tid < cnt) {
         const uint32_t m = (uint32_t)p.members[mbase + tid];
-        s_dest[tid] = (int)((m >> 16) * p.n_used + (m & 0xFFFFu));
+        const uint32_t t = m >> 16, slot = m & 0xFFFFu;
+        s_dest[tid] = (int)(slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot);
     }
 
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    const uint8_t *wrow = p.down + (uint64_t)e * p.dbpe + (uint64_t)(row0 + r) * nb * kSuperBytes;
+    const uint8_t *wrow = (extra ? p.sh_down : p.down + (uint64_t)e * p.dbpe) +
+                          (uint64_t)(row0 + r) * nb * kSuperBytes;
     uint32_t sb = wave;
     WSuper w0 = {}, w1 = {};
     if (sb < nb) w0 = load_wsuper(wrow + (uint64_t)sb * kSuperBytes, kb);
