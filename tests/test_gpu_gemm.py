@@ -59,7 +59,7 @@ def test_gemm_path_without_shared_expert():
 
 
 def test_gemm_path_all_tokens_on_the_same_experts_and_empty_slots():
-    """Worst-case imbalance: every token picks experts {0..3}; several full 64-column tiles
+    """Worst-case imbalance: every token picks experts {0..3}; a full 128-column tile
     per expert plus a ragged one.  A few slots are empty (-1)."""
     s = H.Shape(1024, 512, 16, 4, clamp=10.0, seed=93)
     T = 150
@@ -100,3 +100,40 @@ def test_config2_v3_shape_T256_takes_the_gemm_path_by_default():
     hw = H.host_weights(s, experts=np.unique(sel_h[pick]))
     want = ref.moe_forward(hw, x[pick], sel_h[pick], w_h[pick])
     assert H.max_rel(out.cpu().numpy()[pick], want) < OUT_TOL
+
+
+def test_config3_v3_shape_T4096_zipf_routing():
+    """BASELINE config 3 at its full size.  Checked three ways: the routing of all 4096 tokens
+    against the oracle; a sample of tokens against the oracle's layer; and the size-independent
+    property that a token's output does not depend on its batch -- 64 tokens taken out of the
+    4096 and run on their own (by-expert path, T=64) must give the rows they had in the batch."""
+    s = H.CFG2
+    T = 4096
+    shift = 0.416 * H.zipf_logit_shift(s.n_expert, 3)  # top 10 % of the experts get ~50 % of the picks
+    x, logits, bias = H.host_inputs(s, T, shift)
+    dw = H.device_weights(s)
+    layer = MoeLayer(dw, T)
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    out, sel, w = layer.run(dx, dl, want_routing=True)
+    torch.cuda.synchronize()
+    out_h, sel_h, w_h = out.cpu().numpy(), sel.cpu().numpy(), w.cpu().numpy()
+    cnt = np.bincount(sel_h.ravel(), minlength=s.n_expert)
+    assert np.sort(cnt)[::-1][:26].sum() > 0.4 * cnt.sum()     # the skew is there
+    assert cnt.max() > 8 * 128                                  # several full column tiles
+
+    rsel, _ = H.oracle_route(s, logits, bias)
+    _, scores = ref.router_scores(logits, bias, s.router_mode, s.n_group, s.topk_group)
+    assert H.routing_mismatch_explained(sel_h, rsel, scores, s.n_used) == []
+
+    pick = np.array([0, 1365, 2730, 4095])
+    hw = H.host_weights(s, experts=np.unique(sel_h[pick]))
+    want = ref.moe_forward(hw, x[pick], sel_h[pick], w_h[pick])
+    assert H.max_rel(out_h[pick], want) < OUT_TOL
+
+    sub = np.arange(17, T, 64)[:64]
+    small = MoeLayer(dw, 64)
+    got = small.run(torch.from_numpy(x[sub]).cuda(), None,
+                    selected_in=torch.from_numpy(sel_h[sub]).cuda(),
+                    weights_in=torch.from_numpy(w_h[sub]).cuda())
+    torch.cuda.synchronize()
+    assert H.max_rel(out_h[sub], got.cpu().numpy()) < BASE_TOL
