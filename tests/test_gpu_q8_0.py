@@ -188,3 +188,37 @@ def test_q8_0_shape_contract():
     with pytest.raises(capi.DsxError) as e:   # k = 96: not a multiple of 128
         dispatch.moe_gate_up_batch(FMT_Q8_0, f, z, z, z, f, i, 102, 102, 1, 0.0, 16, 3)
     assert e.value.code == capi.ERR_SHAPE
+
+
+def test_config5_full_size_T512_adversarial_and_uniform_routing():
+    """BASELINE config 5 at its full size (T=512).  Adversarial routing (every token on experts
+    0..7: 512 members per group) and uniform routing; a sample of tokens against the oracle and,
+    as the size-independent check, 16 tokens taken out of the batch and run on their own."""
+    s, T = H.CFG5, 512
+    rng = np.random.default_rng(55)
+    x, logits, bias = H.host_inputs(s, T)
+    w = rng.uniform(0.05, 0.6, (T, 8)).astype(np.float32)
+    dw = H.device_weights(s)
+    layer = MoeLayer(dw, T)
+    small = MoeLayer(dw, 16)
+    dx = torch.from_numpy(x).cuda()
+    cases = {
+        "adversarial": np.tile(np.arange(8, dtype=np.int32), (T, 1)),
+        "uniform": np.stack([rng.choice(s.n_expert, 8, replace=False) for _ in range(T)]).astype(np.int32),
+    }
+    for name, sel in cases.items():
+        out = layer.run(dx, None, selected_in=torch.from_numpy(sel).cuda(),
+                        weights_in=torch.from_numpy(w).cuda())
+        torch.cuda.synchronize()
+        out_h = out.cpu().numpy()
+        pick = np.array([0, 255, 511])
+        hw = H.host_weights(s, experts=np.unique(sel[pick]))
+        want = ref.moe_forward(hw, x[pick], sel[pick], w[pick])
+        assert H.max_rel(out_h[pick], want) < OUT_TOL, name
+        sub = np.arange(3, T, 32)[:16]
+        got = small.run(torch.from_numpy(x[sub]).cuda(), None,
+                        selected_in=torch.from_numpy(sel[sub]).cuda(),
+                        weights_in=torch.from_numpy(w[sub]).cuda())
+        torch.cuda.synchronize()
+        # the same kernels and the same per-column arithmetic: only the chunking differs
+        assert H.max_rel(out_h[sub], got.cpu().numpy()) < 1e-5, name
