@@ -48,8 +48,8 @@ struct GemmParams {
     const uint8_t *act;            // staged activation rows, act_row_bytes apart
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
     const float *ew;               // [n_tokens, n_used]               (gate/up)
-    uint8_t *midq;                 // staged rows out, out_row_bytes   (gate/up)
-    float *mid;                    // f32 [dest rows, n_rows] or null  (gate/up, checking aid)
+    uint8_t *midq;                 // staged rows out, out_row_bytes, or null (gate/up)
+    float *mid;                    // f32 [dest rows, n_rows] or null  (gate/up)
     float *partials;               // f32 [dest rows, n_rows]          (down)
     uint32_t n_tokens, n_used, n_expert;
     uint32_t n_rows;               // weight rows of one matrix
@@ -382,6 +382,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
             }
         }
     }
+    if (p.midq == nullptr) return;  // f32 mid only (a down matrix of another format follows)
     __syncthreads();
     const uint32_t n_blk_out = p.n_rows / 256u;
     if (tid < (uint32_t)kGemmMT) {

@@ -220,5 +220,7 @@ def test_config5_full_size_T512_adversarial_and_uniform_routing():
                         selected_in=torch.from_numpy(sel[sub]).cuda(),
                         weights_in=torch.from_numpy(w[sub]).cuda())
         torch.cuda.synchronize()
-        # the same kernels and the same per-column arithmetic: only the chunking differs
-        assert H.max_rel(out_h[sub], got.cpu().numpy()) < 1e-5, name
+        # the batch takes the grouped GEMM for gate/up, the 16 tokens the by-expert kernel: the
+        # same integer dots summed in a different f32 order, so a mid value next to a rounding
+        # boundary of the Q8_0 quantization may move one int8 step
+        assert H.max_rel(out_h[sub], got.cpu().numpy()) < 1e-3, name
