@@ -167,6 +167,18 @@ def test_mixed_precision_small_layer():
         assert H.max_rel(out, want) < OUT_TOL
 
 
+@pytest.mark.parametrize("T", [128, 131, 300])
+def test_mixed_precision_many_tokens_take_the_grouped_gemms(T):
+    """From 128 tokens on: MXFP4 gate/up GEMM with f32 mid rows, Q8_0 rows, int8-MFMA down GEMM
+    (groups of more than 128 members at T=300: two column tiles, the second ragged)."""
+    s = H.Shape(512, 256, 8, 2, FMT_MXFP4, FMT_Q8_0, clamp=10.0, seed=36, route_scale=2.5)
+    out, want = layer_case(s, T)
+    assert H.max_rel(out, want) < OUT_TOL
+    s = H.Shape(1024, 512, 16, 4, FMT_MXFP4, FMT_Q8_0, shared=False, seed=37)
+    out, want = layer_case(s, T)
+    assert H.max_rel(out, want) < OUT_TOL
+
+
 def test_config5_mixed_precision_adversarial_and_uniform_routing():
     """BASELINE config 5 (gate/up MXFP4, down Q8_0, V3 shape) at a reduced token count: every
     token on experts 0..7, then uniform random distinct top-8."""
