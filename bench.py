@@ -117,6 +117,37 @@ def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
             "mfma_frac_useful_vs_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK}
 
 
+def mixed_leg(H, torch, np, T=512):
+    """BASELINE config 5: MXFP4 gate/up, Q8_0 down, V3 shape, T = 512; every token on experts
+    0..7 (worst-case imbalance) and uniform random distinct top-8."""
+    from deepstrix_amd.executor import MoeLayer
+    s = H.CFG5
+    rng = np.random.default_rng(55)
+    x, _, _ = H.host_inputs(s, T)
+    layer = MoeLayer(H.device_weights(s), T)
+    dx = torch.from_numpy(x).cuda()
+    dw = torch.from_numpy(rng.uniform(0.05, 0.6, (T, s.n_used)).astype(np.float32)).cuda()
+    out = torch.empty((T, s.hidden), dtype=torch.float32, device="cuda")
+    cases = {"adversarial": np.tile(np.arange(s.n_used, dtype=np.int32), (T, 1)),
+             "uniform": np.stack([rng.choice(s.n_expert, s.n_used, replace=False)
+                                  for _ in range(T)]).astype(np.int32)}
+    res = {"tokens": T}
+    for name, sel in cases.items():
+        ds = torch.from_numpy(sel).cuda()
+        for _ in range(2):
+            layer.run(dx, None, out=out, selected_in=ds, weights_in=dw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps = 8
+        for _ in range(reps):
+            layer.run(dx, None, out=out, selected_in=ds, weights_in=dw)
+        torch.cuda.synchronize()
+        res[f"{name}_ms_per_layer"] = (time.perf_counter() - t0) / reps * 1e3
+    del layer
+    torch.cuda.empty_cache()
+    return res
+
+
 def chain_leg(H, torch, np, n_layers=8, T=2, steps=256):
     """BASELINE config 4: 8 chained V3-shape MXFP4 layers, each h += MoE(RMSNorm(h)), T = 2
     tokens per step, 256 consecutive steps with fresh N(0,1) inputs.  Latency of one step from
@@ -261,6 +292,8 @@ def main():
         extra["prefill_T4096"] = prefill_leg(layers[0].w, base, H, torch, np)
     if not args.no_chain:
         extra["chain_8_layers_T2"] = chain_leg(H, torch, np)
+    if not args.no_extra:
+        extra["mixed_precision_T512_cfg5"] = mixed_leg(H, torch, np)
 
     result = {
         "metric": "moe_layer_us_per_token_T1",

@@ -247,12 +247,15 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     for (uint32_t i = qb * kRouterThreads + tid; i < p.n_counters; i += (gridDim.x - n_route) * kRouterThreads)
         p.counters[i] = 0;
-    const uint32_t blk = qb * 4u + (tid >> 6);
-    if (blk >= p.n_tokens * p.n_sb) return;
-    const uint32_t t = blk / p.n_sb, b = blk - t * p.n_sb;
-    const float4 v = *(const float4 *)(p.x + (uint64_t)t * p.n_sb * 256u + (size_t)b * 256u + lane * 4u);
-    uint8_t *row = p.xp + (uint64_t)t * p.xp_row_bytes;
-    quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
+    // one wave per 256-element block, grid-stride (many tokens: a few thousand workgroups
+    // instead of one per four blocks)
+    const uint32_t n_q = gridDim.x - n_route;
+    for (uint32_t blk = qb * 4u + (tid >> 6); blk < p.n_tokens * p.n_sb; blk += n_q * 4u) {
+        const uint32_t t = blk / p.n_sb, b = blk - t * p.n_sb;
+        const float4 v = *(const float4 *)(p.x + (uint64_t)t * p.n_sb * 256u + (size_t)b * 256u + lane * 4u);
+        uint8_t *row = p.xp + (uint64_t)t * p.xp_row_bytes;
+        quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
+    }
 }
 
 // Rows of f32 -> staged rows (the mid activations of the by-expert path).
