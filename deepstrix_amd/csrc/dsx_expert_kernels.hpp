@@ -130,6 +130,10 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t row0 = blockIdx.x * 16u;
     const uint32_t item = blockIdx.y;
+    // decode from a staged row that one pass of the workgroup covers: loaded before the weights
+    const bool early = !BY_EXPERT && STAGED && NT == 1 && p.n_blocks * 32u <= 4u * kGuWaves * 64u;
+    uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {};
+    float early_yd = 0.0f;
 
     // ---- which expert, which columns -------------------------------------------------
     const uint8_t *gate_e, *up_e;
@@ -159,6 +163,17 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         cnt = 1;
         const uint32_t n_slots = p.n_used + (p.sh_gate ? 1u : 0u);
         const uint32_t t = item / n_slots, slot = item - t * n_slots;
+        if (STAGED && early) {
+            // the token's staged row goes out first: it needs nothing but the token index, and
+            // (loads of a wave return in order) it must not queue behind the weights
+            const uint8_t *xrow = p.xq + (uint64_t)t * p.xq_row_bytes;
+            const uint32_t nq = p.n_blocks * 32u, q = tid, step = kGuWaves * 64u;
+            if (q < nq) ex0 = *(const uint4 *)(xrow + (size_t)q * 16u);
+            if (q + step < nq) ex1 = *(const uint4 *)(xrow + (size_t)(q + step) * 16u);
+            if (q + 2u * step < nq) ex2 = *(const uint4 *)(xrow + (size_t)(q + 2u * step) * 16u);
+            if (q + 3u * step < nq) ex3 = *(const uint4 *)(xrow + (size_t)(q + 3u * step) * 16u);
+            if (tid < p.n_blocks) early_yd = *((const float *)(xrow + (size_t)p.n_blocks * 512u) + tid);
+        }
         if (slot < p.n_used) {
             const int e = p.selected[t * p.n_used + slot];
             if (e < 0) {  // empty slot: defined output, nothing to compute
@@ -205,7 +220,15 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
 
     // ---- activations into LDS -----------------------------------------------------------
     __syncthreads();  // s_tok visible
-    if (STAGED) {
+    if (STAGED && early) {
+        // (NT == 1: the row's tile bytes are contiguous in LDS as they are in memory)
+        const uint32_t nq = p.n_blocks * 32u, q = tid, step = kGuWaves * 64u;
+        if (q < nq) *(uint4 *)(tiles + (size_t)q * 16u) = ex0;
+        if (q + step < nq) *(uint4 *)(tiles + (size_t)(q + step) * 16u) = ex1;
+        if (q + 2u * step < nq) *(uint4 *)(tiles + (size_t)(q + 2u * step) * 16u) = ex2;
+        if (q + 3u * step < nq) *(uint4 *)(tiles + (size_t)(q + 3u * step) * 16u) = ex3;
+        if (tid < p.n_blocks) s_yd[tid] = early_yd;
+    } else if (STAGED) {
         if (BY_EXPERT)
             stage_copy<NT, kGuWaves * 64>(tiles, s_yd, cnt, p.n_blocks, tid,
                                           StageMembers{p.xq, p.xq_row_bytes, s_tok});
@@ -357,6 +380,30 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
         return base + row_off + (uint64_t)b * kSuperBytes;
     };
 
+    // The activation rows go out first when five loads per thread cover them: they need only
+    // the token index, and (a wave's loads return in order) must not queue behind the weights.
+    const uint32_t per_slot = nb * 32u;                 // 16-byte pieces of one slot's tiles
+    const uint32_t n_pieces = p.n_slots * per_slot;
+    constexpr uint32_t kStep = kDownWaves * 64u;
+    const bool early = STAGED && n_pieces <= 5u * kStep && units <= kStep;
+    uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {}, ex4 = {};
+    float early_yd = 0.0f;
+    auto piece_src = [&](uint32_t q) -> const uint8_t * {
+        const uint32_t j = q / per_slot, c = q - j * per_slot;
+        return xq + (uint64_t)j * p.xq_slot_stride + (size_t)c * 16u;
+    };
+    if (early) {
+        if (tid < n_pieces) ex0 = *(const uint4 *)piece_src(tid);
+        if (tid + kStep < n_pieces) ex1 = *(const uint4 *)piece_src(tid + kStep);
+        if (tid + 2u * kStep < n_pieces) ex2 = *(const uint4 *)piece_src(tid + 2u * kStep);
+        if (tid + 3u * kStep < n_pieces) ex3 = *(const uint4 *)piece_src(tid + 3u * kStep);
+        if (tid + 4u * kStep < n_pieces) ex4 = *(const uint4 *)piece_src(tid + 4u * kStep);
+        if (tid < units) {
+            const uint32_t j = tid / nb, bq = tid - j * nb;
+            early_yd = *((const float *)(xq + (uint64_t)j * p.xq_slot_stride + (size_t)nb * 512u) + bq);
+        }
+    }
+
     // five (slot, super-block) units of weights in flight per wave
     uint32_t un = wave;
     WSuper w0 = {}, w1 = {}, w2 = {}, w3 = {}, w4 = {};
@@ -367,7 +414,15 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     if (un + 4 * kDownWaves < units && live) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
 
     if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? selected[tid] : 0;
-    if (STAGED) {
+    if (early) {
+        // (a slot's tiles are contiguous in LDS as they are in its row)
+        if (tid < n_pieces) *(uint4 *)(tiles + (size_t)tid * 16u) = ex0;
+        if (tid + kStep < n_pieces) *(uint4 *)(tiles + (size_t)(tid + kStep) * 16u) = ex1;
+        if (tid + 2u * kStep < n_pieces) *(uint4 *)(tiles + (size_t)(tid + 2u * kStep) * 16u) = ex2;
+        if (tid + 3u * kStep < n_pieces) *(uint4 *)(tiles + (size_t)(tid + 3u * kStep) * 16u) = ex3;
+        if (tid + 4u * kStep < n_pieces) *(uint4 *)(tiles + (size_t)(tid + 4u * kStep) * 16u) = ex4;
+        if (tid < units) s_yd[tid] = early_yd;
+    } else if (STAGED) {
         stage_copy<1, kDownWaves * 64>(tiles, s_yd, p.n_slots, nb, tid,
                                        StageSlots{xq, p.xq_slot_stride, nb});
     } else {
