@@ -217,8 +217,9 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
                                      void *down_end);
 /* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens: from this many tokens on, an all-MXFP4 layer runs the grouped-GEMM path
- * (64 token columns per work item, shared expert as an extra group).
+ * gemm_min_tokens: from this many tokens on, a layer with MXFP4 gate/up runs the grouped-GEMM
+ * path (128 token columns per work item, shared expert as an extra group; a Q8_0 down matrix
+ * takes the int8 grouped GEMM).
  * decode_max_tokens: up to this many tokens, an all-MXFP4 layer runs the one-token decode
  * kernels once per token inside the same launches (no grouping by expert). */
 int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
