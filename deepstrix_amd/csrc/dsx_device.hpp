@@ -136,6 +136,8 @@ __device__ __forceinline__ void stage_q8k_block(uint8_t *tile, float *yd_slot,
 // vector register holds the data.  They count in vmcnt like any load; the compiler does not
 // see them, so the caller waits (s_waitcnt vmcnt) before the LDS reads that depend on them.
 // `base` must be uniform; `off` is the lane's unsigned byte offset from it.
+// Each helper overwrites M0 (the compiler has no clobber name for it); the kernels that use them
+// contain nothing else that needs M0 (no LDS-direct builtins, no indirect register indexing).
 __device__ __forceinline__ void lds_dma16(uint32_t lds_addr, const void *base, uint32_t off) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
