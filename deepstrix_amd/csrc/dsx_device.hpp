@@ -61,23 +61,28 @@ __device__ __forceinline__ uint32_t gload4(const uint8_t *p) {
     return *(const DSX_GLOBAL uint32_t *)(uintptr_t)p;
 }
 
-// E4M3 (OCP) byte of a small non-negative integer m in [0, 15].
-__device__ __forceinline__ uint32_t e4m3_of_uint(uint32_t m) {
-    // 0,1,2,3,4,5,6,7 -> 0x00,0x38,0x40,0x44,0x48,0x4A,0x4C,0x4E ; 8..15 -> 0x50 | (m & 7)
-    const uint32_t lo = 0x44403800u, hi = 0x4E4C4A48u;
-    const uint32_t t = (m & 4u) ? hi : lo;
-    const uint32_t small = (t >> ((m & 3u) * 8u)) & 0xFFu;
-    return (m & 8u) ? (0x50u | (m & 7u)) : small;
-}
-
-// int8 q -> (high plane byte, low plane byte):  q = 16 * hi + lo, hi in [-8, 7], lo in [0, 15].
-__device__ __forceinline__ void split_q(int q, uint32_t &hi_byte, uint32_t &lo_byte) {
-    const uint32_t u = (uint32_t)(q + 128) & 0xFFu;
-    const uint32_t ul = u & 15u, uh = u >> 4;
-    lo_byte = e4m3_of_uint(ul);
-    const bool neg = uh < 8u;
-    const uint32_t mag = neg ? (8u - uh) : (uh - 8u);
-    hi_byte = e4m3_of_uint(mag) | (neg ? 0x80u : 0u);
+// int8 q -> (high plane byte, low plane byte):  q + 128 = 16 * uh + ul, the high plane holds
+// uh - 8 in [-8, 7], the low plane ul in [0, 15], both as E4M3 (OCP) bytes:
+// 0,1,..,7 -> 0x00,0x38,0x40,0x44,0x48,0x4A,0x4C,0x4E ; 8..15 -> 0x50 | (m & 7); sign in bit 7.
+// Four int8 values at once (one per byte of `q`, any order) -> the dwords of the high and of the
+// low plane with the same byte order.  Bytewise table look-ups (v_perm_b32) instead of four
+// scalar splits: u = q + 128 = q ^ 0x80, low nibble and high nibble each index a 16-entry
+// table of E4M3 bytes, taken as two 8-entry halves selected by the nibble's bit 3.
+__device__ __forceinline__ void split_q4(uint32_t q, uint32_t &hi_word, uint32_t &lo_word) {
+    const uint32_t u = q ^ 0x80808080u;
+    const uint32_t ul = u & 0x0F0F0F0Fu, uh = (u >> 4) & 0x0F0F0F0Fu;
+    // E4M3 of 0..7 and of 8..15; E4M3 of -(8 - m) for m = 0..7
+    constexpr uint32_t kPos03 = 0x44403800u, kPos47 = 0x4E4C4A48u;
+    constexpr uint32_t kBig03 = 0x53525150u, kBig47 = 0x57565554u;
+    constexpr uint32_t kNeg03 = 0xCACCCED0u, kNeg47 = 0xB8C0C4C8u;
+    const uint32_t sl = ul & 0x07070707u, sh = uh & 0x07070707u;
+    const uint32_t ml = ((ul >> 3) & 0x01010101u) * 0xFFu, mh = ((uh >> 3) & 0x01010101u) * 0xFFu;
+    const uint32_t lo_small = __builtin_amdgcn_perm(kPos47, kPos03, sl);
+    const uint32_t lo_big = __builtin_amdgcn_perm(kBig47, kBig03, sl);
+    lo_word = (lo_big & ml) | (lo_small & ~ml);
+    const uint32_t hi_neg = __builtin_amdgcn_perm(kNeg47, kNeg03, sh);   // uh < 8: value uh - 8 < 0
+    const uint32_t hi_pos = __builtin_amdgcn_perm(kPos47, kPos03, sh);   // uh >= 8: value uh - 8
+    hi_word = (hi_pos & mh) | (hi_neg & ~mh);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -115,15 +120,10 @@ __device__ __forceinline__ void stage_q8k_block(uint8_t *tile, float *yd_slot,
     const int8_t *q8 = (const int8_t *)(blk + 4) + b32 * 32u;
     const uint16_t lo2 = *(const uint16_t *)(q8 + 2u * d);
     const uint16_t hi2 = *(const uint16_t *)(q8 + 16u + 2u * d);
-    const int q0 = (int8_t)(lo2 & 0xFF), q2 = (int8_t)(lo2 >> 8);
-    const int q1 = (int8_t)(hi2 & 0xFF), q3 = (int8_t)(hi2 >> 8);
-    uint32_t h0, l0, h1, l1, h2, l2, h3, l3;
-    split_q(q0, h0, l0);
-    split_q(q1, h1, l1);
-    split_q(q2, h2, l2);
-    split_q(q3, h3, l3);
-    const uint32_t hw = h0 | (h1 << 8) | (h2 << 16) | (h3 << 24);
-    const uint32_t lw = l0 | (l1 << 8) | (l2 << 16) | (l3 << 24);
+    // nibble positions 4d..4d+3 = elements (2d, 16+2d, 2d+1, 17+2d)
+    const uint32_t packed = __builtin_amdgcn_perm((uint32_t)hi2, (uint32_t)lo2, 0x05010400u);
+    uint32_t hw, lw;
+    split_q4(packed, hw, lw);
     const uint32_t h = b32 >> 2, b = b32 & 3u;
     const uint32_t c = b >> 1, kb = 2u * (b & 1u) + (d >> 2), o = (d & 3u) * 4u;
     *(uint32_t *)(tile + tile_off<NT>(h, 0, c, kb, col) + o) = hw;

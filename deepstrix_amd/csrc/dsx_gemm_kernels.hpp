@@ -412,7 +412,8 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
         const float iscale = s_iscale[col];
 #pragma unroll
         for (int rho = 0; rho < kGemmRF / 2; rho++) {
-            uint32_t hw[2] = {0u, 0u}, lw[2] = {0u, 0u};
+            // dword q / 2 of a plane holds bytes 2 * (q & 1) + rr
+            uint32_t qw[2] = {0u, 0u};
 #pragma unroll
             for (int rr = 0; rr < 2; rr++) {
                 const v4f v4 = acc[2 * rho + rr][0][j];
@@ -422,13 +423,12 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                     int qi = (int)rintf(iscale * v);
                     qi = qi > 127 ? 127 : qi;
                     qi = qi < -128 ? -128 : qi;
-                    uint32_t hb, lb;
-                    split_q(qi, hb, lb);
-                    const uint32_t sh = (uint32_t)(2 * (q & 1) + rr) * 8u;
-                    hw[q >> 1] |= hb << sh;
-                    lw[q >> 1] |= lb << sh;
+                    qw[q >> 1] |= ((uint32_t)qi & 0xFFu) << ((uint32_t)(2 * (q & 1) + rr) * 8u);
                 }
             }
+            uint32_t hw[2], lw[2];
+            split_q4(qw[0], hw[0], lw[0]);
+            split_q4(qw[1], hw[1], lw[1]);
             if (col >= cnt) continue;
             const uint32_t b32 = wave * (kGemmRF / 2) + rho;
             const uint32_t hh = b32 >> 2, bb = b32 & 3u;

@@ -95,16 +95,11 @@ __device__ __forceinline__ void quantize_block_to_staged(float4 v, uint32_t lane
     const bool low_half = m < 4u;                   // holds elements < 16 of the block
     const uint32_t lo4 = low_half ? mine : other;   // elements 4mm .. 4mm+3
     const uint32_t hi4 = low_half ? other : mine;   // elements 16+4mm .. 16+4mm+3
-    const uint32_t sh = low_half ? 0u : 16u;        // low-half lane: first two; other: last two
-    const int qa = (int8_t)((lo4 >> sh) & 0xFF), qc = (int8_t)((lo4 >> (sh + 8u)) & 0xFF);
-    const int qb = (int8_t)((hi4 >> sh) & 0xFF), qd = (int8_t)((hi4 >> (sh + 8u)) & 0xFF);
-    uint32_t h0, l0, h1, l1, h2, l2, h3, l3;
-    split_q(qa, h0, l0);
-    split_q(qb, h1, l1);
-    split_q(qc, h2, l2);
-    split_q(qd, h3, l3);
-    const uint32_t hw = h0 | (h1 << 8) | (h2 << 16) | (h3 << 24);
-    const uint32_t lw = l0 | (l1 << 8) | (l2 << 16) | (l3 << 24);
+    // low-half lane: the first two of each group of four; other: the last two.  Packed in the
+    // order of the tile dword's nibble positions (a, b, c, d) = (lo4[k], hi4[k], lo4[k+1], hi4[k+1])
+    const uint32_t packed = __builtin_amdgcn_perm(hi4, lo4, low_half ? 0x05010400u : 0x07030602u);
+    uint32_t hw, lw;
+    split_q4(packed, hw, lw);
     const uint32_t b32 = lane >> 3, d = 2u * (m & 3u) + (low_half ? 0u : 1u);
     const uint32_t h = b32 >> 2, b = b32 & 3u;
     const uint32_t c = b >> 1, kb = 2u * (b & 1u) + (d >> 2), o = (d & 3u) * 4u;
