@@ -339,24 +339,34 @@ int dsx_moe_down_batched(dsx_stream_t stream, int dtype, float *out, const uint8
 }
 
 // ---- by-expert ------------------------------------------------------------------------
-int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,
-                        int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
-                        const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
-                        uint32_t chunk) {
+// extra: also build group n_expert that holds every token (slot n_used)
+static int group_build_impl(hipStream_t st, int32_t *group_count, int32_t *group_offset,
+                            int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
+                            const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
+                            uint32_t chunk, bool extra) {
     if (!group_count || !group_offset || !expert_members || !work_items || !n_work_items || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_group_build: null pointer");
     if (n_expert == 0 || n_expert > DSX_MAX_EXPERTS)
         return fail(DSX_ERR_INVALID_ARG, "moe_group_build: n_expert=%u", n_expert);
     if (b >= 65536 || n_used == 0 || n_used >= 65536)
         return fail(DSX_ERR_INVALID_ARG, "moe_group_build: b=%u n_used=%u must be below 65536", b, n_used);
-    if (chunk == 0 || chunk > 64) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..64", chunk);
+    if (chunk == 0 || chunk > 128) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..128", chunk);
     if ((uint64_t)b * n_used > 2048u)  // many picks: histogram launch + one workgroup per expert
-        return group_build_big(S(stream), group_count, group_offset, expert_members, work_items,
-                               n_work_items, selected, b, n_used, n_expert, chunk, false);
-    hipLaunchKernelGGL(k_group_build, dim3(1), dim3(kGbThreads), 0, S(stream), group_count,
+        return group_build_big(st, group_count, group_offset, expert_members, work_items,
+                               n_work_items, selected, b, n_used, n_expert, chunk, extra);
+    hipLaunchKernelGGL(k_group_build, dim3(1), dim3(kGbThreads), 0, st, group_count,
                        group_offset, expert_members, work_items, n_work_items, selected, b, n_used,
-                       n_expert, chunk);
+                       n_expert, chunk, extra ? 1u : 0u);
     return launched("moe_group_build");
+}
+
+int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,
+                        int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
+                        const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
+                        uint32_t chunk) {
+    if (chunk > 64) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..64", chunk);
+    return group_build_impl(S(stream), group_count, group_offset, expert_members, work_items,
+                            n_work_items, selected, b, n_used, n_expert, chunk, false);
 }
 
 static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,

@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kGbThreads) void k_group_build(
     int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
     int32_t *__restrict__ members, int32_t *__restrict__ work_items,
     int32_t *__restrict__ n_work_items, const int32_t *__restrict__ selected, uint32_t b,
-    uint32_t n_used, uint32_t n_expert, uint32_t chunk) {
+    uint32_t n_used, uint32_t n_expert, uint32_t chunk, uint32_t extra) {
     __shared__ int s_count[DSX_MAX_EXPERTS_K];
     __shared__ int s_off[DSX_MAX_EXPERTS_K + 1];
     __shared__ int s_wi_off[DSX_MAX_EXPERTS_K + 1];
@@ -363,9 +363,20 @@ __global__ __launch_bounds__(kGbThreads) void k_group_build(
         }
         s_off[n_expert] = acc;
         s_wi_off[n_expert] = wacc;
-        *n_work_items = wacc;
+        // the optional extra group n_expert: every token, slot n_used
+        *n_work_items = wacc + (extra ? (int)((b + chunk - 1) / chunk) : 0);
     }
     __syncthreads();
+    if (extra) {
+        const uint32_t base = (uint32_t)s_off[n_expert], wbase = (uint32_t)s_wi_off[n_expert];
+        for (uint32_t t = tid; t < b; t += kGbThreads) members[base + t] = (int)((t << 16) | n_used);
+        for (uint32_t c = tid; c < (b + chunk - 1) / chunk; c += kGbThreads)
+            work_items[wbase + c] = (int)((n_expert << 16) | (c * chunk));
+        if (tid == 0) {
+            group_count[n_expert] = (int)b;
+            group_offset[n_expert + 1] = (int)(base + b);
+        }
+    }
     for (uint32_t e = tid; e < n_expert; e += kGbThreads) {
         group_count[e] = s_count[e];
         group_offset[e] = s_off[e];
