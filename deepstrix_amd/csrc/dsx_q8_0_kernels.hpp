@@ -374,41 +374,54 @@ inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *d
 
 
 // ---------------------------------------------------------------------------------------
-// down for many tokens per expert: a grouped GEMM on the int8 matrix instruction.
+// Expert products for many tokens per expert: grouped GEMMs on the int8 matrix instruction.
 // Work item = (expert, first member), the next up to 128 members are the token columns; a
 // workgroup (4 waves) multiplies 64 weight rows with them over all k, wave w owning rows
-// 16 w .. 16 w + 15 and all columns (8 accumulator fragments).  One
-// v_mfma_i32_16x16x32_i8 is exactly one Q8_0 block of a 16 x 16 fragment; its int32 sums are
-// folded into the f32 accumulators with f16(d_w) * xscale, as in q8_0_row_partial.
+// 16 w .. 16 w + 15 and all columns.
+//   gate/up (PAIR):  the 64 rows of gate and the same 64 rows of up; the epilogue applies the
+//                    clamped SwiGLU and the routing weight and stores f32 mid rows;
+//   down:            f32 partial rows, one per (token, slot).
+// One v_mfma_i32_16x16x32_i8 is exactly one Q8_0 block of a 16 x 16 fragment; its int32 sums
+// are folded into the f32 accumulators with f16(d_w) * xscale, as in q8_0_row_partial.
 // Operands are fetched in memory order by LDS-direct loads (see lds_dma16) in chunks of 4
 // blocks (128 k), double buffered: the weights into a region private to the wave, the
 // activations (and their scales) shared; 16-byte units are XOR-swizzled with the row so
-// that the 8-byte operand reads spread over the banks.  f32 partial rows out, one per
-// (token, slot); the extra expert (index n_expert, slot n_used) like in the MXFP4 GEMM.
-// LDS: B[2][16 KB] | xs[2][2 KB] | A[4 waves][2][2 KB] | dw[64 rows][n_blocks] f16
+// that the 8-byte operand reads spread over the banks.  The extra expert (index n_expert,
+// slot n_used) like in the MXFP4 GEMM.
+// LDS: B[2][16 KB] | xs[2][2 KB] | A[4 waves][M][2][2 KB] | dw[M][64 rows][n_blocks] f16,
+// M = 2 matrices for PAIR, else 1.
 // ---------------------------------------------------------------------------------------
 constexpr int kQgWaves = 4;
 constexpr int kQgCols = 128;
 constexpr int kQgRows = 64;
-constexpr uint32_t kQgBOff = 0, kQgXsOff = 2 * 16384, kQgAOff = kQgXsOff + 2 * 2048,
-                   kQgDwOff = kQgAOff + kQgWaves * 2 * 2048;
+constexpr uint32_t kQgBOff = 0, kQgXsOff = 2 * 16384, kQgAOff = kQgXsOff + 2 * 2048;
 
 struct Q8GemmParams {
-    float *partials;               // f32 [dest rows, n_rows]
-    const uint8_t *w, *sh_w;       // [n_expert] experts; the extra expert or null
-    uint64_t bpe;
-    const uint8_t *act;            // Q8_0 activation rows, act_row_bytes apart, indexed by dest row
+    float *out;                    // PAIR: f32 mid [dest rows, n_rows]; else partials [dest rows, n_rows]
+    const uint8_t *w0, *w1;        // [n_expert] experts: gate and up, or down in w0
+    const uint8_t *sh_w0, *sh_w1;  // the extra expert, or null
+    uint64_t bpe0, bpe1;
+    const uint8_t *act;            // Q8_0 activation rows, act_row_bytes apart: by token (PAIR) or dest row
+    const float *ew;               // [n_tokens, n_used]   (PAIR)
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
     uint32_t n_tokens, n_used, n_expert, n_rows, n_blocks, act_row_bytes, n_row_tiles;
+    float clamp, sh_clamp;
 };
 
-inline size_t q8_0_gemm_lds_bytes(uint32_t n_blocks) { return kQgDwOff + (size_t)kQgRows * n_blocks * 2u; }
+inline size_t q8_0_gemm_lds_bytes(uint32_t n_blocks, bool pair) {
+    const uint32_t m = pair ? 2u : 1u;
+    return kQgAOff + (size_t)kQgWaves * m * 4096u + (size_t)m * kQgRows * n_blocks * 2u;
+}
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm_down(const Q8GemmParams p) {
+template <bool PAIR>
+__global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams p) {
+    constexpr uint32_t M = PAIR ? 2u : 1u;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ uint32_t s_dest[kQgCols];
+    __shared__ uint32_t s_src[kQgCols];
+    __shared__ float s_ew[kQgCols];
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t g4 = lane >> 4, n16 = lane & 15u;
@@ -428,44 +441,53 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm_down(const Q8GemmPa
     const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
     const uint32_t cnt = min((uint32_t)kQgCols, (uint32_t)p.group_count[e] - start);
     const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+    const bool extra = e >= p.n_expert;
     if (tid < (uint32_t)kQgCols) {
         // columns past the end of the group repeat its last member; they are never stored
         const uint32_t m = (uint32_t)p.members[mbase + min(tid, cnt - 1u)];
         const uint32_t t = m >> 16, slot = m & 0xFFFFu;
-        s_dest[tid] = slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot;
+        const uint32_t dest = slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot;
+        s_dest[tid] = dest;
+        s_src[tid] = PAIR ? t : dest;
+        if (PAIR) s_ew[tid] = slot >= p.n_used ? 1.0f : p.ew[dest];
     }
     const uint32_t nb = p.n_blocks, row_bytes = nb * 34u;
-    const uint8_t *wbase = (e >= p.n_expert ? p.sh_w : p.w + (uint64_t)e * p.bpe) +
-                           (uint64_t)(rt * kQgRows) * row_bytes;
+    const uint8_t *wbase[M];
+    wbase[0] = (extra ? p.sh_w0 : p.w0 + (uint64_t)e * p.bpe0) + (uint64_t)(rt * kQgRows) * row_bytes;
+    if (PAIR) wbase[M - 1] = (extra ? p.sh_w1 : p.w1 + (uint64_t)e * p.bpe1) + (uint64_t)(rt * kQgRows) * row_bytes;
 
-    // the 64 rows' block scales, once: dw[row][block]
-    uint16_t *s_dw = (uint16_t *)(smem + kQgDwOff);
-    for (uint32_t i = tid; i < (uint32_t)kQgRows * nb; i += kQgWaves * 64u) {
-        const uint32_t r = i / nb, b = i - r * nb;
-        s_dw[i] = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(wbase + (uint64_t)r * row_bytes + b * 2u);
+    // the 64 rows' block scales of each matrix, once: dw[matrix][row][block]
+    const uint32_t dw_off = kQgAOff + kQgWaves * M * 4096u;
+    uint16_t *s_dw = (uint16_t *)(smem + dw_off);
+    for (uint32_t i = tid; i < M * (uint32_t)kQgRows * nb; i += kQgWaves * 64u) {
+        const uint32_t mm = i / ((uint32_t)kQgRows * nb), j = i - mm * (uint32_t)kQgRows * nb;
+        const uint32_t r = j / nb, b = j - r * nb;
+        s_dw[i] = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(wbase[PAIR ? mm : 0] + (uint64_t)r * row_bytes + b * 2u);
     }
-    __syncthreads();  // s_dest visible
+    __syncthreads();  // s_src visible
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t l8 = lane >> 3, c8 = (lane & 7u) ^ l8;
-    // A: wave w, rows 16 w + 8 i + l8, 16-byte unit c8 of the chunk's 128 bytes
-    const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + kQgAOff + wave * 4096u);
+    // A: wave w, matrix mm, rows 16 w + 8 i + l8, 16-byte unit c8 of the chunk's 128 bytes
+    const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + kQgAOff + wave * M * 4096u);
     const uint32_t a_fetch = (wave * 16u + l8) * row_bytes + nb * 2u + c8 * 16u;
     // B: wave w fetches columns 32 w + 8 ii + l8
     const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + kQgBOff + wave * 4096u);
     uint32_t b_fetch[4];
 #pragma unroll
     for (int ii = 0; ii < 4; ii++)
-        b_fetch[ii] = s_dest[wave * 32u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
+        b_fetch[ii] = s_src[wave * 32u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
     // activation scales: waves 0 and 1, lane -> column 64 w + lane, the chunk's 4 floats
     const uint32_t xs_lds = __builtin_amdgcn_readfirstlane(lds0 + kQgXsOff + (wave & 1u) * 1024u);
-    const uint32_t xs_fetch = s_dest[(wave & 1u) * 64u + lane] * p.act_row_bytes + nb * 32u;
+    const uint32_t xs_fetch = s_src[(wave & 1u) * 64u + lane] * p.act_row_bytes + nb * 32u;
     const bool b_live = wave * 32u < cnt;
     auto issue = [&](uint32_t c, uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
-            lds_dma16(a_lds + buf * 2048u + (uint32_t)i * 1024u, wbase,
-                      a_fetch + (uint32_t)i * 8u * row_bytes + c * 128u);
+        for (uint32_t mm = 0; mm < M; mm++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                lds_dma16(a_lds + mm * 4096u + buf * 2048u + (uint32_t)i * 1024u, wbase[mm],
+                          a_fetch + (uint32_t)i * 8u * row_bytes + c * 128u);
         if (b_live) {
 #pragma unroll
             for (int ii = 0; ii < 4; ii++)
@@ -477,13 +499,15 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm_down(const Q8GemmPa
     // read side: lane (row / column n16, 8-byte piece g4 of a block's 32 bytes)
     const uint32_t rd = (n16 >> 3) * 1024u + (n16 & 7u) * 128u + (g4 & 1u) * 8u;
     const uint32_t rd_sw = n16 & 7u, rd_unit = g4 >> 1;
-    const uint8_t *a_ptr = smem + kQgAOff + wave * 4096u;
+    const uint8_t *a_ptr = smem + kQgAOff + wave * M * 4096u;
 
-    float acc[8][4];
+    float acc[M][8][4];
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (uint32_t mm = 0; mm < M; mm++)
 #pragma unroll
-        for (int q = 0; q < 4; q++) acc[j][q] = 0.0f;
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) acc[mm][j][q] = 0.0f;
 
     const uint32_t n_chunks = nb / 4u;
     const uint32_t nj = (cnt + 15u) / 16u;
@@ -493,22 +517,26 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm_down(const Q8GemmPa
     for (uint32_t c = 0; c < n_chunks; c++) {
         const uint32_t buf = c & 1u;
         if (c + 1u < n_chunks) issue(c + 1u, buf ^ 1u);
-        const uint8_t *ab = a_ptr + buf * 2048u, *bb = smem + kQgBOff + buf * 16384u;
+        const uint8_t *bb = smem + kQgBOff + buf * 16384u;
         const uint8_t *xb = smem + kQgXsOff + buf * 2048u;
-        // the lane's 4 rows' scales of the chunk's 4 blocks
-        float dw[4][4];
+        // the lane's 4 rows' scales of the chunk's 4 blocks, and its A operands
+        float dw[M][4][4];
+        long av[M][4];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint2 h = *(const uint2 *)(s_dw + (size_t)(wave * 16u + g4 * 4u + q) * nb + c * 4u);
-            dw[q][0] = __half2float(__ushort_as_half((uint16_t)(h.x & 0xFFFFu)));
-            dw[q][1] = __half2float(__ushort_as_half((uint16_t)(h.x >> 16)));
-            dw[q][2] = __half2float(__ushort_as_half((uint16_t)(h.y & 0xFFFFu)));
-            dw[q][3] = __half2float(__ushort_as_half((uint16_t)(h.y >> 16)));
+        for (uint32_t mm = 0; mm < M; mm++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint2 h = *(const uint2 *)(s_dw + (size_t)(mm * kQgRows + wave * 16u + g4 * 4u + q) * nb + c * 4u);
+                dw[mm][q][0] = __half2float(__ushort_as_half((uint16_t)(h.x & 0xFFFFu)));
+                dw[mm][q][1] = __half2float(__ushort_as_half((uint16_t)(h.x >> 16)));
+                dw[mm][q][2] = __half2float(__ushort_as_half((uint16_t)(h.y & 0xFFFFu)));
+                dw[mm][q][3] = __half2float(__ushort_as_half((uint16_t)(h.y >> 16)));
+            }
+            const uint8_t *ab = a_ptr + mm * 4096u + buf * 2048u;
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                av[mm][b] = *(const long *)(ab + rd + (((uint32_t)(2 * b) + rd_unit) ^ rd_sw) * 16u);
         }
-        long av[4];
-#pragma unroll
-        for (int b = 0; b < 4; b++)
-            av[b] = *(const long *)(ab + rd + (((uint32_t)(2 * b) + rd_unit) ^ rd_sw) * 16u);
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             if ((uint32_t)j < nj) {  // uniform
@@ -518,11 +546,14 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm_down(const Q8GemmPa
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
                     const long bv = *(const long *)(bj + (((uint32_t)(2 * b) + rd_unit) ^ rd_sw) * 16u);
-                    const v4i32 s = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], bv, v4i32{0, 0, 0, 0}, 0, 0, 0);
-                    acc[j][0] += dw[0][b] * xsv[b] * (float)s.x;
-                    acc[j][1] += dw[1][b] * xsv[b] * (float)s.y;
-                    acc[j][2] += dw[2][b] * xsv[b] * (float)s.z;
-                    acc[j][3] += dw[3][b] * xsv[b] * (float)s.w;
+#pragma unroll
+                    for (uint32_t mm = 0; mm < M; mm++) {
+                        const v4i32 s = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[mm][b], bv, v4i32{0, 0, 0, 0}, 0, 0, 0);
+                        acc[mm][j][0] += dw[mm][0][b] * xsv[b] * (float)s.x;
+                        acc[mm][j][1] += dw[mm][1][b] * xsv[b] * (float)s.y;
+                        acc[mm][j][2] += dw[mm][2][b] * xsv[b] * (float)s.z;
+                        acc[mm][j][3] += dw[mm][3][b] * xsv[b] * (float)s.w;
+                    }
                 }
             }
         }
@@ -531,31 +562,41 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm_down(const Q8GemmPa
     }
 
     // the lane holds rows 16 w + 4 g4 + q of columns 16 j + n16
+    const float clamp = extra ? p.sh_clamp : p.clamp;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const uint32_t col = j * 16u + n16;
         if (col >= cnt) continue;
-        float *dst = p.partials + (uint64_t)s_dest[col] * p.n_rows + rt * kQgRows + wave * 16u + g4 * 4u;
-        *(float4 *)dst = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        float *dst = p.out + (uint64_t)s_dest[col] * p.n_rows + rt * kQgRows + wave * 16u + g4 * 4u;
+        if (PAIR) {
+            const float ew = s_ew[col];
+            *(float4 *)dst = make_float4(swiglu_clamp(acc[0][j][0], acc[M - 1][j][0], clamp, ew),
+                                         swiglu_clamp(acc[0][j][1], acc[M - 1][j][1], clamp, ew),
+                                         swiglu_clamp(acc[0][j][2], acc[M - 1][j][2], clamp, ew),
+                                         swiglu_clamp(acc[0][j][3], acc[M - 1][j][3], clamp, ew));
+        } else {
+            *(float4 *)dst = make_float4(acc[0][j][0], acc[0][j][1], acc[0][j][2], acc[0][j][3]);
+        }
     }
 }
 
-inline int q8_0_gemm_down(hipStream_t st, const Q8GemmParams &p, uint32_t max_wi) {
+template <bool PAIR>
+inline int q8_0_gemm(hipStream_t st, const Q8GemmParams &p, uint32_t max_wi) {
     if (max_wi == 0) return DSX_OK;
     if (p.n_rows % kQgRows || p.n_blocks % 4 || p.n_blocks == 0)
         return q8_0_fail(DSX_ERR_SHAPE, "q8_0 gemm", "n_rows must be a multiple of 64, k of 128");
     const uint64_t act_rows = (uint64_t)p.n_tokens * (p.n_used + 1u);
     if ((uint64_t)p.n_rows * p.n_blocks * 34u > 0xFFFFFFFFull || act_rows * p.act_row_bytes > 0xFFFFFFFFull)
         return q8_0_fail(DSX_ERR_INVALID_ARG, "q8_0 gemm", "a weight matrix or the activation rows exceed 4 GiB");
-    const size_t lds = q8_0_gemm_lds_bytes(p.n_blocks);
+    const size_t lds = q8_0_gemm_lds_bytes(p.n_blocks, PAIR);
     if (lds > 140 * 1024) return q8_0_fail(DSX_ERR_UNSUPPORTED, "q8_0 gemm", "k too large for the scale table in LDS");
     const uint32_t per_xcd = (max_wi + 7u) / 8u;
     const uint64_t grid = (uint64_t)8u * per_xcd * p.n_row_tiles;
     if (grid > 0x7FFFFFFFull) return q8_0_fail(DSX_ERR_INVALID_ARG, "q8_0 gemm", "grid too large");
-    static const hipError_t attr = hipFuncSetAttribute((const void *)k_q8_0_gemm_down,
+    static const hipError_t attr = hipFuncSetAttribute((const void *)k_q8_0_gemm<PAIR>,
                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
     (void)attr;
-    hipLaunchKernelGGL(k_q8_0_gemm_down, dim3((uint32_t)grid), dim3(kQgWaves * 64), lds, st, p);
+    hipLaunchKernelGGL(k_q8_0_gemm<PAIR>, dim3((uint32_t)grid), dim3(kQgWaves * 64), lds, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? DSX_OK : q8_0_fail((int)e, "q8_0 gemm", hipGetErrorString(e));
 }

@@ -141,6 +141,26 @@ def test_config1_q8_0_layer(T):
     assert H.max_rel(out, want) < OUT_TOL
 
 
+@pytest.mark.parametrize("T", [128, 300])
+def test_config1_shape_many_tokens_take_the_int8_grouped_gemms(T):
+    """An all-Q8_0 layer from 128 tokens on: gate/up (SwiGLU in the epilogue) and down as
+    int8-MFMA grouped GEMMs, the shared expert as the extra group."""
+    out, want = layer_case(H.CFG1, T)
+    assert H.max_rel(out, want) < OUT_TOL
+
+
+def test_small_q8_0_layer_many_tokens_skewed_groups():
+    """Groups of more than 128 members (two column tiles, the second ragged), empty experts."""
+    s = H.Shape(512, 256, 8, 2, FMT_Q8_0, FMT_Q8_0, clamp=5.0, seed=38)
+    T = 200
+    rng = np.random.default_rng(38)
+    sel = np.stack([rng.choice(3, 2, replace=False) for _ in range(T)]).astype(np.int32)  # experts 0..2 only
+    sel[7, 1] = -1
+    w = rng.uniform(0.1, 1.0, (T, 2)).astype(np.float32)
+    out, want = layer_case(s, T, sel, w)
+    assert H.max_rel(out, want) < OUT_TOL
+
+
 def test_config1_router_logits_from_fp32_matvec():
     """Config 1 names a router matrix W f32 N(0, 0.02): logits = W . x feed the same layer."""
     s, T = H.CFG1, 4
