@@ -117,6 +117,31 @@ def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
             "mfma_frac_useful_vs_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK}
 
 
+def q8_0_leg(H, torch, np):
+    """BASELINE config 1 (the reference's CPU-runnable case): all-Q8_0 layer, hidden 2048, 64 + 1
+    experts, top-6 softmax, inter 1408, T = 4; and the same layer with 512 tokens."""
+    from deepstrix_amd.executor import MoeLayer
+    s = H.CFG1
+    layer = MoeLayer(H.device_weights(s), 512)
+    res = {}
+    for T in (4, 512):
+        x, logits, _ = H.host_inputs(s, T)
+        dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+        out = torch.empty((T, s.hidden), dtype=torch.float32, device="cuda")
+        for _ in range(3):
+            layer.run(dx, dl, out=out)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps = 20
+        for _ in range(reps):
+            layer.run(dx, dl, out=out)
+        torch.cuda.synchronize()
+        res[f"T{T}_us_per_layer"] = (time.perf_counter() - t0) / reps * 1e6
+    del layer
+    torch.cuda.empty_cache()
+    return res
+
+
 def mixed_leg(H, torch, np, T=512):
     """BASELINE config 5: MXFP4 gate/up, Q8_0 down, V3 shape, T = 512; every token on experts
     0..7 (worst-case imbalance) and uniform random distinct top-8."""
@@ -294,6 +319,7 @@ def main():
         extra["chain_8_layers_T2"] = chain_leg(H, torch, np)
     if not args.no_extra:
         extra["mixed_precision_T512_cfg5"] = mixed_leg(H, torch, np)
+        extra["q8_0_cfg1"] = q8_0_leg(H, torch, np)
 
     result = {
         "metric": "moe_layer_us_per_token_T1",

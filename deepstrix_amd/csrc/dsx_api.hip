@@ -388,7 +388,8 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     if (dtype == DSX_FMT_Q8_0)
         return q8_0_gate_up_by_expert(S(stream), mid, gate, up, xq, ew, group_count, group_offset,
                                       expert_members, work_items, n_work_items, max_work_items,
-                                      gbpe, ubpe, n_used, chunk, clamp, n_rows, n_blocks);
+                                      gbpe, ubpe, n_used, chunk, clamp, n_rows, n_blocks, sh_gate, sh_up,
+                                      sh_clamp, n_expert, n_tokens);
     if (dtype != DSX_FMT_MXFP4)
         return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows: no kernel for dtype %d", dtype);
     if (n_rows == 0 || n_rows % 16 != 0)
@@ -451,7 +452,8 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
     if (dtype == DSX_FMT_Q8_0)
         return q8_0_down_by_expert(S(stream), partials, down, xq, group_count, group_offset,
                                    expert_members, work_items, n_work_items, max_work_items, dbpe,
-                                   xq_slot_stride, n_used, chunk, n_rows, n_blocks_in);
+                                   xq_slot_stride, n_used, chunk, n_rows, n_blocks_in, sh_down, n_expert,
+                                   n_tokens);
     if (dtype != DSX_FMT_MXFP4)
         return fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert: no kernel for dtype %d", dtype);
     if (n_rows == 0 || n_rows % 16 != 0)

@@ -42,6 +42,8 @@ struct Q8Params {
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
     uint32_t x_stride, n_used, chunk, n_rows, n_blocks;
     float clamp, sh_clamp;
+    // by-expert with the extra expert (index n_expert, slot n_used; rows after the routed ones)
+    uint32_t n_expert, n_tokens;
 };
 
 // The lane's share of `row . x[c]` for NT columns, over all of its blocks.
@@ -119,11 +121,13 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_gate_up(const Q8Params p
             const uint32_t m = (uint32_t)p.members[mbase + tid];
             const uint32_t t = m >> 16, slot = m & 0xFFFFu;
             s_tok[tid] = t;
-            s_dest[tid] = t * p.n_used + slot;
-            s_ew[tid] = p.ew[t * p.n_used + slot];
+            s_dest[tid] = slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot;
+            s_ew[tid] = slot >= p.n_used ? 1.0f : p.ew[t * p.n_used + slot];
         }
-        g_e = p.w0 + (uint64_t)e * p.bpe0;
-        u_e = p.w1 + (uint64_t)e * p.bpe1;
+        const bool extra = p.sh_w0 != nullptr && e >= p.n_expert;
+        g_e = extra ? p.sh_w0 : p.w0 + (uint64_t)e * p.bpe0;
+        u_e = extra ? p.sh_w1 : p.w1 + (uint64_t)e * p.bpe1;
+        if (extra) clamp = p.sh_clamp;
     } else {
         if (item < p.n_used) {
             const int e = p.selected[item];
@@ -222,13 +226,14 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_by_expert(const Q8P
     const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
     if (tid < cnt) {
         const uint32_t m = (uint32_t)p.members[mbase + tid];
-        s_dest[tid] = (m >> 16) * p.n_used + (m & 0xFFFFu);
+        const uint32_t t = m >> 16, slot = m & 0xFFFFu;
+        s_dest[tid] = slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot;
     }
     __syncthreads();
     q8_0_stage(lds_x, cnt, row_bytes, tid,
                [&](uint32_t j) { return p.xq + (uint64_t)s_dest[j] * p.x_stride; });
     __syncthreads();
-    const uint8_t *w_e = p.w0 + (uint64_t)e * p.bpe0;
+    const uint8_t *w_e = (p.sh_w0 != nullptr && e >= p.n_expert) ? p.sh_w0 : p.w0 + (uint64_t)e * p.bpe0;
     const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
     for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
         const uint32_t row = row0 + r;
@@ -319,7 +324,9 @@ inline int q8_0_gate_up_by_expert(hipStream_t st, float *mid, const uint8_t *gat
                                   const int32_t *group_offset, const int32_t *members,
                                   const int32_t *work_items, const int32_t *n_work_items,
                                   uint32_t max_wi, uint64_t gbpe, uint64_t ubpe, uint32_t n_used,
-                                  uint32_t chunk, float clamp, uint32_t n_rows, uint32_t n_blocks) {
+                                  uint32_t chunk, float clamp, uint32_t n_rows, uint32_t n_blocks,
+                                  const uint8_t *sh_gate = nullptr, const uint8_t *sh_up = nullptr,
+                                  float sh_clamp = 0.0f, uint32_t n_expert = 0, uint32_t n_tokens = 0) {
     if (chunk > 8) return q8_0_fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows", "Q8_0 takes chunk <= 8");
     const int nt = q8_0_pick_nt(chunk);
     int rc = q8_0_check("moe_gate_up_chunked_rows", n_rows, n_blocks, gate, up, gbpe, ubpe, xq,
@@ -331,6 +338,7 @@ inline int q8_0_gate_up_by_expert(hipStream_t st, float *mid, const uint8_t *gat
     p.work_items = work_items; p.n_work_items = n_work_items;
     p.x_stride = q8_0_act_row_bytes(n_blocks); p.n_used = n_used; p.chunk = chunk; p.n_rows = n_rows;
     p.n_blocks = n_blocks; p.clamp = clamp;
+    p.sh_w0 = sh_gate; p.sh_w1 = sh_up; p.sh_clamp = sh_clamp; p.n_expert = n_expert; p.n_tokens = n_tokens;
     const dim3 grid(n_rows / kQ8RowsPerWg, max_wi), block(kQ8Waves * 64);
     const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks);
     switch (nt) {
@@ -348,7 +356,8 @@ inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *d
                                const int32_t *members, const int32_t *work_items,
                                const int32_t *n_work_items, uint32_t max_wi, uint64_t dbpe,
                                uint32_t xq_slot_stride, uint32_t n_used, uint32_t chunk,
-                               uint32_t n_rows, uint32_t n_blocks_in) {
+                               uint32_t n_rows, uint32_t n_blocks_in, const uint8_t *sh_down = nullptr,
+                               uint32_t n_expert = 0, uint32_t n_tokens = 0) {
     if (chunk > 8) return q8_0_fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert", "Q8_0 takes chunk <= 8");
     const int nt = q8_0_pick_nt(chunk);
     int rc = q8_0_check("moe_down_by_expert", n_rows, n_blocks_in, down, nullptr, dbpe, 0, xq,
@@ -360,6 +369,7 @@ inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *d
     p.work_items = work_items; p.n_work_items = n_work_items;
     p.x_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk; p.n_rows = n_rows;
     p.n_blocks = n_blocks_in;
+    p.sh_w0 = sh_down; p.n_expert = n_expert; p.n_tokens = n_tokens;
     const dim3 grid(n_rows / kQ8RowsPerWg, max_wi), block(kQ8Waves * 64);
     const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks_in);
     switch (nt) {
