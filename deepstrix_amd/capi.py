@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(PKG, "lib", "libdsx_moe.so")
 
 FMT_Q8_0 = 8
 FMT_MXFP4 = 39
+SRC_F32, SRC_BF16, SRC_F8E4M3 = 0, 1, 2  # dsx_q8_0_weights_from_hf source types
 ROUTER_SQRT_SOFTPLUS, ROUTER_SIGMOID, ROUTER_SOFTMAX = 0, 1, 2
 ERR_INVALID_ARG, ERR_SHAPE, ERR_UNSUPPORTED, ERR_DEVICE = -1, -2, -3, -4
 Q8K_BLOCK_BYTES = 292
@@ -72,6 +73,8 @@ SIGNATURES = {
     "dsx_rms_norm": (_int, [_vp, _vp, _vp, _vp, _u32, _f32, _u32]),
     "dsx_swiglu_clamp_weighted": (_int, [_vp, _vp, _vp, _vp, _vp, _f32, _u32, _u32]),
     "dsx_mxfp4_repack_hf_to_v2": (_int, [_vp, _vp, _vp, _vp, _u32, _u32]),
+    "dsx_q8_0_weights_from_hf": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32]),
+    "dsx_q8_0_repack_rows": (_int, [_vp, _vp, _vp, _u32, _u32]),
     "dsx_dequant_rows": (_int, [_vp, _int, _vp, _vp, _u32, _u32]),
     "dsx_moe_layer_create": (_int, [C.POINTER(LayerDesc), C.POINTER(_vp)]),
     "dsx_moe_layer_destroy": (None, [_vp]),

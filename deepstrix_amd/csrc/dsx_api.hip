@@ -571,6 +571,62 @@ int dsx_mxfp4_repack_hf_to_v2(dsx_stream_t stream, uint8_t *dst, const uint8_t *
     return launched("mxfp4_repack");
 }
 
+int dsx_q8_0_weights_from_hf(dsx_stream_t stream, uint8_t *dst, const void *src,
+                             const uint8_t *scale, uint32_t src_dtype, uint32_t out_rows,
+                             uint32_t in_cols, uint32_t scale_rows, uint32_t scale_cols,
+                             uint32_t split_rows) {
+    if (out_rows == 0 || in_cols == 0) return DSX_OK;
+    if (!dst || !src) return fail(DSX_ERR_INVALID_ARG, "q8_0_weights_from_hf: null pointer");
+    if (in_cols % 32 != 0)
+        return fail(DSX_ERR_SHAPE, "q8_0_weights_from_hf: in_cols=%u must be a multiple of 32", in_cols);
+    if (!aligned(dst, 2)) return fail(DSX_ERR_SHAPE, "q8_0_weights_from_hf: dst must be 2-byte aligned");
+    uint32_t br = 1, bc = 1;
+    const uint64_t groups = (uint64_t)out_rows * (in_cols / 32) * 8;
+    const dim3 grid((uint32_t)((groups + 255) / 256));
+    if (groups > 0xFFFFFFFFull * 256ull) return fail(DSX_ERR_SHAPE, "q8_0_weights_from_hf: matrix too large");
+    switch (src_dtype) {
+    case DSX_SRC_F32:
+        if (!aligned(src, 16)) return fail(DSX_ERR_SHAPE, "q8_0_weights_from_hf: f32 src must be 16-byte aligned");
+        hipLaunchKernelGGL(k_q8_0_weights<kSrcF32>, grid, dim3(256), 0, S(stream), dst, src, scale,
+                           out_rows, in_cols, br, bc, 1u, split_rows);
+        break;
+    case DSX_SRC_BF16:
+        if (!aligned(src, 8)) return fail(DSX_ERR_SHAPE, "q8_0_weights_from_hf: bf16 src must be 8-byte aligned");
+        hipLaunchKernelGGL(k_q8_0_weights<kSrcBF16>, grid, dim3(256), 0, S(stream), dst, src, scale,
+                           out_rows, in_cols, br, bc, 1u, split_rows);
+        break;
+    case DSX_SRC_F8E4M3:
+        if (!scale) return fail(DSX_ERR_INVALID_ARG, "q8_0_weights_from_hf: fp8 weight without a scale tensor");
+        if (scale_rows == 0 || scale_cols == 0 || out_rows % scale_rows != 0 || in_cols % scale_cols != 0)
+            return fail(DSX_ERR_SHAPE,
+                        "q8_0_weights_from_hf: fp8 scale grid %ux%u does not exactly tile %ux%u",
+                        scale_rows, scale_cols, out_rows, in_cols);
+        if (!aligned(src, 4)) return fail(DSX_ERR_SHAPE, "q8_0_weights_from_hf: fp8 src must be 4-byte aligned");
+        br = out_rows / scale_rows;
+        bc = in_cols / scale_cols;
+        hipLaunchKernelGGL(k_q8_0_weights<kSrcF8E4M3>, grid, dim3(256), 0, S(stream), dst, src, scale,
+                           out_rows, in_cols, br, bc, scale_cols, split_rows);
+        break;
+    default:
+        return fail(DSX_ERR_INVALID_ARG, "q8_0_weights_from_hf: cannot Q8_0-quantise source dtype %u", src_dtype);
+    }
+    return launched("q8_0_weights_from_hf");
+}
+
+int dsx_q8_0_repack_rows(dsx_stream_t stream, uint8_t *dst, const uint8_t *src, uint32_t num_rows,
+                         uint32_t blocks_per_row) {
+    if (num_rows == 0 || blocks_per_row == 0) return DSX_OK;
+    if (!dst || !src) return fail(DSX_ERR_INVALID_ARG, "q8_0_repack_rows: null pointer");
+    if (dst == src) return fail(DSX_ERR_INVALID_ARG, "q8_0_repack_rows: cannot repack in place");
+    if (!aligned(dst, 2) || !aligned(src, 2))
+        return fail(DSX_ERR_SHAPE, "q8_0_repack_rows: dst and src must be 2-byte aligned");
+    const uint64_t groups = (uint64_t)num_rows * blocks_per_row * 8;
+    if (groups > 0xFFFFFFFFull * 256ull) return fail(DSX_ERR_SHAPE, "q8_0_repack_rows: matrix too large");
+    hipLaunchKernelGGL(k_q8_0_repack_rows, dim3((uint32_t)((groups + 255) / 256)), dim3(256), 0,
+                       S(stream), dst, src, num_rows, blocks_per_row);
+    return launched("q8_0_repack_rows");
+}
+
 int dsx_dequant_rows(dsx_stream_t stream, int dtype, float *y, const uint8_t *rows, uint32_t n_rows,
                      uint32_t cols) {
     if (n_rows == 0 || cols == 0) return DSX_OK;

@@ -793,6 +793,114 @@ __global__ __launch_bounds__(256) void k_q8_0_dequant(float *__restrict__ y,
     for (int j = 0; j < 32; j++) y[i * 32u + j] = d * (float)q[j];
 }
 
+// ---------------------------------------------------------------------------------------
+// Checkpoint matrix -> Q8_0 weights.  Source values are f32, bf16, or fp8-e4m3 codes times an
+// E8M0 scale grid whose cells are br x bc elements; eight lanes share a 32-element block
+// (four elements each).  d = amax/127 in f32 stored as f16 (round to nearest even),
+// q = round-half-away(x * (1/d)), NaN -> 0.
+// crates/v4flash-core/src/hf_v41.rs:728-805 (read_q8), :99-118 (E8M0, E4M3), :125-137 (block).
+// split != 0 writes engine rows [blocks x f16 d][blocks x 32 i8]
+// (crates/v4flash-kernels/src/weights.rs:225-240), else ggml blocks [f16 d][32 i8].
+// ---------------------------------------------------------------------------------------
+constexpr uint32_t kSrcF32 = 0u, kSrcBF16 = 1u, kSrcF8E4M3 = 2u;
+
+__device__ __forceinline__ float e4m3_value(uint32_t b) {  // torch float8_e4m3fn
+    if ((b & 0x7Fu) == 0x7Fu) return __uint_as_float(0x7FC00000u);
+    const uint32_t e = (b >> 3) & 15u, m = b & 7u;
+    const float v = (e == 0u) ? (float)m * 0x1p-9f
+                              : (1.0f + (float)m * 0.125f) * __uint_as_float((e + 120u) << 23);
+    return (b & 0x80u) ? -v : v;
+}
+__device__ __forceinline__ float e8m0_value(uint32_t e) {  // torch float8_e8m0fnu
+    if (e == 0xFFu) return __uint_as_float(0x7FC00000u);
+    return __uint_as_float(e == 0u ? (1u << 22) : (e << 23));
+}
+
+__device__ __forceinline__ void store_q4(uint8_t *p, uint32_t packed) {
+    if (((uintptr_t)p & 3u) == 0u) {
+        *(uint32_t *)p = packed;
+    } else {
+        *(uint16_t *)p = (uint16_t)packed;
+        *(uint16_t *)(p + 2) = (uint16_t)(packed >> 16);
+    }
+}
+
+template <uint32_t SRC>
+__global__ __launch_bounds__(256) void k_q8_0_weights(uint8_t *__restrict__ dst,
+                                                      const void *__restrict__ src,
+                                                      const uint8_t *__restrict__ scale,
+                                                      uint32_t out_rows, uint32_t in_cols,
+                                                      uint32_t br, uint32_t bc, uint32_t sc,
+                                                      uint32_t split) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint32_t bpr = in_cols / 32u;
+    const uint64_t blk = gid >> 3;
+    const uint32_t sub = (uint32_t)(gid & 7u);
+    const bool live = blk < (uint64_t)out_rows * bpr;
+    const uint64_t r = live ? blk / bpr : 0, b = live ? blk - r * bpr : 0;
+    const uint64_t c0 = b * 32u + sub * 4u;
+    float xs[4] = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        if (SRC == kSrcF32) {
+            const float4 v = *(const float4 *)((const float *)src + r * in_cols + c0);
+            xs[0] = v.x, xs[1] = v.y, xs[2] = v.z, xs[3] = v.w;
+        } else if (SRC == kSrcBF16) {
+            const uint2 v = *(const uint2 *)((const uint16_t *)src + r * in_cols + c0);
+            xs[0] = __uint_as_float(v.x << 16), xs[1] = __uint_as_float(v.x & 0xFFFF0000u);
+            xs[2] = __uint_as_float(v.y << 16), xs[3] = __uint_as_float(v.y & 0xFFFF0000u);
+        } else {
+            const uint32_t v = *(const uint32_t *)((const uint8_t *)src + r * in_cols + c0);
+            const uint8_t *srow = scale + (r / br) * sc;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                xs[i] = e4m3_value((v >> (8 * i)) & 0xFFu) * e8m0_value(srow[(c0 + i) / bc]);
+        }
+    }
+    // fmaxf drops NaN operands, like the reference's fold over f32::max
+    float amax = fmaxf(fmaxf(fmaxf(0.0f, fabsf(xs[0])), fabsf(xs[1])),
+                       fmaxf(fabsf(xs[2]), fabsf(xs[3])));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    if (!live) return;
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float t = roundf(xs[i] * id);
+        int q = (t != t) ? 0 : (t >= 127.0f ? 127 : (t <= -128.0f ? -128 : (int)t));
+        packed |= (uint32_t)(q & 0xFF) << (8 * i);
+    }
+    uint8_t *dp, *qp;
+    if (split) {
+        uint8_t *row = dst + r * bpr * 34u;
+        dp = row + b * 2u;
+        qp = row + (uint64_t)bpr * 2u + b * 32u + sub * 4u;
+    } else {
+        dp = dst + blk * 34u;
+        qp = dp + 2u + sub * 4u;
+    }
+    store_q4(qp, packed);
+    if (sub == 0) *(__half *)dp = __float2half_rn(d);
+}
+
+// ggml Q8_0 blocks -> engine rows (crates/v4flash-kernels/src/weights.rs:225-240).
+__global__ __launch_bounds__(256) void k_q8_0_repack_rows(uint8_t *__restrict__ dst,
+                                                          const uint8_t *__restrict__ src,
+                                                          uint32_t n_rows, uint32_t bpr) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t blk = gid >> 3;
+    const uint32_t sub = (uint32_t)(gid & 7u);
+    if (blk >= (uint64_t)n_rows * bpr) return;
+    const uint64_t r = blk / bpr, b = blk - r * bpr;
+    const uint8_t *s = src + blk * 34u;
+    uint8_t *row = dst + r * bpr * 34u;
+    const uint32_t lo = *(const uint16_t *)(s + 2u + sub * 4u), hi = *(const uint16_t *)(s + 4u + sub * 4u);
+    store_q4(row + (uint64_t)bpr * 2u + b * 32u + sub * 4u, lo | (hi << 16));
+    if (sub == 0) *(uint16_t *)(row + b * 2u) = *(const uint16_t *)s;
+}
+
 // Identity grouping for a dense expert: every token is a member of expert 0 with weight 1.
 __global__ __launch_bounds__(256) void k_dense_groups(int32_t *__restrict__ group_count,
                                                       int32_t *__restrict__ group_offset,

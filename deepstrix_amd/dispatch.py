@@ -149,6 +149,22 @@ def mxfp4_repack_hf_to_v2(dst, packed, scale, out, nb):
     check(lib().dsx_mxfp4_repack_hf_to_v2(_stream(), _p(dst), _p(packed), _p(scale), out, nb))
 
 
+def q8_0_weights_from_hf(dst, src, scale, src_dtype, out_rows, in_cols, split_rows=True):
+    """A checkpoint matrix (f32, bf16 or fp8-e4m3 + E8M0 scale grid) -> Q8_0 weights
+    (crates/v4flash-core/src/hf_v41.rs:728-805; split rows as
+    crates/v4flash-kernels/src/weights.rs:225-240 lays them out)."""
+    capi.init()
+    sr, sc = (scale.shape if scale is not None else (0, 0))
+    check(lib().dsx_q8_0_weights_from_hf(_stream(), _p(dst), _p(src), _p(scale), src_dtype, out_rows,
+                                         in_cols, sr, sc, 1 if split_rows else 0))
+
+
+def q8_0_repack_rows(dst, src, num_rows, blocks_per_row):
+    """crates/v4flash-kernels/src/weights.rs:225-240"""
+    capi.init()
+    check(lib().dsx_q8_0_repack_rows(_stream(), _p(dst), _p(src), num_rows, blocks_per_row))
+
+
 def dequant_rows(dt, y, rows, n_rows, cols):
     capi.init()
     check(lib().dsx_dequant_rows(_stream(), dt, _p(y), _p(rows), n_rows, cols))

@@ -179,6 +179,24 @@ int dsx_swiglu_clamp_weighted(dsx_stream_t stream, float *mid, const float *gate
  * HF packed[out, nb*16] + scale[out, nb] -> v2 rows dst[out, nb*17]. nb % 8 == 0. */
 int dsx_mxfp4_repack_hf_to_v2(dsx_stream_t stream, uint8_t *dst, const uint8_t *packed,
                               const uint8_t *scale, uint32_t out, uint32_t nb);
+/* HfV41Source::read_q8 (crates/v4flash-core/src/hf_v41.rs:728-805): a checkpoint matrix
+ * src[out_rows, in_cols] -- f32, bf16, or fp8-e4m3 codes with an E8M0 scale grid
+ * scale[scale_rows, scale_cols] that tiles the matrix exactly (scale is ignored for f32 and
+ * bf16) -- quantized to Q8_0 with quantize_q8_0_block (hf_v41.rs:125-137).  split_rows = 0
+ * writes ggml blocks [f16 d][32 i8] as read_q8 does; split_rows = 1 writes the engine rows
+ * [blocks x f16 d][blocks x 32 i8] that repack_q8_0 makes of them, in one pass.  An fp8
+ * source without scales, or a grid that does not divide the matrix, is refused. */
+#define DSX_SRC_F32 0u
+#define DSX_SRC_BF16 1u
+#define DSX_SRC_F8E4M3 2u
+int dsx_q8_0_weights_from_hf(dsx_stream_t stream, uint8_t *dst, const void *src,
+                             const uint8_t *scale, uint32_t src_dtype, uint32_t out_rows,
+                             uint32_t in_cols, uint32_t scale_rows, uint32_t scale_cols,
+                             uint32_t split_rows);
+/* repack_q8_0 (crates/v4flash-kernels/src/weights.rs:225-240): ggml Q8_0 blocks of a row-major
+ * matrix -> engine rows.  dst and src may not overlap. */
+int dsx_q8_0_repack_rows(dsx_stream_t stream, uint8_t *dst, const uint8_t *src, uint32_t num_rows,
+                         uint32_t blocks_per_row);
 /* Dequantize engine rows to f32 (checking aid; crates/v4flash-core/src/kquants.rs:105-111 for
  * Q8_0, crates/v4flash-kernels/src/mxfp4_tables.rs:38-45 for MXFP4). */
 int dsx_dequant_rows(dsx_stream_t stream, int dtype, float *y, const uint8_t *rows,

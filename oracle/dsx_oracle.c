@@ -243,6 +243,14 @@ void dsx_ref_mxfp4_quantize_v2(const float *x, uint8_t *dst, size_t n_rows, size
 /* Q8_0                                                                      */
 /* ------------------------------------------------------------------------ */
 
+/* Rust's `f32 as i8`: NaN -> 0, out of range saturates. */
+static int8_t sat_i8(float v) {
+    if (v != v) return 0;
+    if (v >= 127.0f) return 127;
+    if (v <= -128.0f) return -128;
+    return (int8_t)v;
+}
+
 /* C/src/hf_v41.rs:125-137: d = amax/127 (f32), id = 1/d, q = round-half-away. */
 void dsx_ref_q8_0_quantize_block(const float *x, uint8_t *out) {
     float amax = 0.0f;
@@ -255,7 +263,7 @@ void dsx_ref_q8_0_quantize_block(const float *x, uint8_t *out) {
     const uint16_t h = dsx_ref_f32_to_f16(d);
     out[0] = (uint8_t)(h & 0xff);
     out[1] = (uint8_t)(h >> 8);
-    for (int i = 0; i < 32; i++) out[2 + i] = (uint8_t)(int8_t)roundf(x[i] * id);
+    for (int i = 0; i < 32; i++) out[2 + i] = (uint8_t)sat_i8(roundf(x[i] * id));
 }
 
 /* K/src/weights.rs:225-240 */
@@ -269,6 +277,39 @@ void dsx_ref_q8_0_repack_rows(const uint8_t *ggml, uint8_t *dst, size_t n_rows, 
             memcpy(d + blocks * 2 + b * 32, s + b * 34 + 2, 32);
         }
     }
+}
+
+/* C/src/hf_v41.rs:728-805 (read_q8): a checkpoint matrix [out, inn] in f32 (dtype 0), bf16
+ * (1) or fp8-e4m3 with an E8M0 scale grid [sr, sc] that tiles it exactly (2) -> ggml Q8_0
+ * blocks (34 B each, row-major).  Returns 0, or -1 where the reference returns Err. */
+int dsx_ref_q8_0_from_hf(const void *src, const uint8_t *scale, int dtype, size_t out, size_t inn,
+                         size_t sr, size_t sc, uint8_t *dst) {
+    if (inn % 32) return -1;
+    size_t br = 0, bc = 0;
+    if (dtype == 2) {
+        if (!scale || sr == 0 || sc == 0) return -1;
+        br = out / sr;
+        bc = inn / sc;
+        if (br * sr != out || bc * sc != inn) return -1;
+    } else if (dtype != 0 && dtype != 1) {
+        return -1;
+    }
+    float *f = (float *)malloc(inn * sizeof(float));
+    for (size_t r = 0; r < out; r++) {
+        for (size_t c = 0; c < inn; c++) {
+            if (dtype == 0)
+                f[c] = ((const float *)src)[r * inn + c];
+            else if (dtype == 1)
+                f[c] = dsx_ref_bf16_to_f32(((const uint16_t *)src)[r * inn + c]);
+            else
+                f[c] = dsx_ref_e4m3_to_f32(((const uint8_t *)src)[r * inn + c]) *
+                       dsx_ref_e8m0_to_f32(scale[(r / br) * sc + c / bc]);
+        }
+        for (size_t b = 0; b < inn / 32; b++)
+            dsx_ref_q8_0_quantize_block(f + b * 32, dst + (r * (inn / 32) + b) * 34);
+    }
+    free(f);
+    return 0;
 }
 
 void dsx_ref_q8_0_quantize_rows(const float *x, uint8_t *dst, size_t n_rows, size_t cols) {

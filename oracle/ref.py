@@ -81,6 +81,8 @@ def _declare(l):
     l.dsx_ref_q8_0_quantize_block.argtypes = [vp, vp]
     l.dsx_ref_q8_0_quantize_rows.argtypes = [vp, vp, sz, sz]
     l.dsx_ref_q8_0_repack_rows.argtypes = [vp, vp, sz, sz]
+    l.dsx_ref_q8_0_from_hf.restype = i32
+    l.dsx_ref_q8_0_from_hf.argtypes = [vp, vp, i32, sz, sz, sz, sz, vp]
     l.dsx_ref_q8_0_dequant_rows.argtypes = [vp, vp, sz, sz]
     l.dsx_ref_q8_0_quantize_act.argtypes = [vp, vp, vp, sz]
     l.dsx_ref_dot_q8_0.restype = f32
@@ -168,6 +170,35 @@ def q8_0_quantize_rows(x: np.ndarray) -> np.ndarray:
     n_rows, cols = x.shape
     dst = np.empty(n_rows * (cols // 32) * 34, np.uint8)
     lib().dsx_ref_q8_0_quantize_rows(_p(x), _p(dst), n_rows, cols)
+    return dst
+
+
+def q8_0_repack_rows(ggml: np.ndarray, n_rows: int, blocks: int) -> np.ndarray:
+    """ggml blocks [d f16 | 32 i8] -> engine rows [blocks x d | blocks x 32 i8]
+    (crates/v4flash-kernels/src/weights.rs:225-240)."""
+    ggml = _c(ggml, np.uint8)
+    dst = np.empty(n_rows * blocks * 34, np.uint8)
+    lib().dsx_ref_q8_0_repack_rows(_p(ggml), _p(dst), n_rows, blocks)
+    return dst
+
+
+SRC_F32, SRC_BF16, SRC_F8E4M3 = 0, 1, 2
+
+
+def q8_0_from_hf(src: np.ndarray, scale: Optional[np.ndarray], dtype: int) -> np.ndarray:
+    """A checkpoint matrix (f32, bf16 bits as uint16, or fp8-e4m3 codes as uint8 with an E8M0
+    scale grid) -> ggml Q8_0 blocks (crates/v4flash-core/src/hf_v41.rs:728-805).  Raises where
+    the reference returns Err."""
+    want = {SRC_F32: np.float32, SRC_BF16: np.uint16, SRC_F8E4M3: np.uint8}[dtype]
+    src = _c(src, want)
+    out, inn = src.shape
+    sr = sc = 0
+    if scale is not None:
+        scale = _c(scale, np.uint8)
+        sr, sc = scale.shape
+    dst = np.empty(out * (inn // 32) * 34, np.uint8)
+    if lib().dsx_ref_q8_0_from_hf(_p(src), _p(scale), dtype, out, inn, sr, sc, _p(dst)) != 0:
+        raise ValueError("q8_0_from_hf: the reference refuses this input")
     return dst
 
 

@@ -219,6 +219,72 @@ def test_q8_0_rows_layout_and_dequant():
         assert np.max(np.abs(y[r] - x[r])) <= np.abs(x[r]).max() / 127 * 0.51 + 1e-6
 
 
+def _q8_0_blocks_numpy(f):
+    """ggml Q8_0 blocks of f32 rows by numpy: d = amax/127 -> float16, q = round half away."""
+    out, inn = f.shape
+    blk = f.reshape(out, inn // 32, 32)
+    amax = np.nanmax(np.abs(np.where(np.isnan(blk), 0, blk)), axis=2).astype(np.float32)
+    d = (amax / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        idv = np.where(d == 0, np.float32(0), np.float32(1.0) / d).astype(np.float32)
+        t = (blk * idv[:, :, None]).astype(np.float32)
+    q = np.where(np.isnan(t), 0, np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)))
+    q = np.clip(q, -128, 127).astype(np.int8)
+    res = np.empty((out, inn // 32, 34), np.uint8)
+    res[:, :, :2] = d.astype(np.float16).view(np.uint8).reshape(out, inn // 32, 2)
+    res[:, :, 2:] = q.view(np.uint8)
+    return res.reshape(-1)
+
+
+def test_q8_0_from_fp8_checkpoint_against_torch_float8_decoders():
+    # crates/v4flash-core/src/hf_v41.rs:728-805; the fp8 / e8m0 values come from torch's own
+    # float8 dtypes (a third-party decoder), the scale grid is indexed here with numpy.repeat
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(21)
+    out, inn, br, bc = 96, 192, 32, 64           # cells are not square: a transposed grid fails
+    codes = rng.integers(0, 256, (out, inn), dtype=np.uint8)
+    scale = rng.integers(110, 140, (out // br, inn // bc), dtype=np.uint8)
+    scale[0, 0] = 255                            # a NaN scale: the whole cell quantizes to zero
+    w = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    sc = torch.from_numpy(scale).view(torch.float8_e8m0fnu).float().numpy()
+    with np.errstate(invalid="ignore"):
+        f = (w * np.repeat(np.repeat(sc, br, axis=0), bc, axis=1)).astype(np.float32)
+    got = ref.q8_0_from_hf(codes, scale, ref.SRC_F8E4M3)
+    assert np.array_equal(got, _q8_0_blocks_numpy(f))
+    assert not got.reshape(out, inn // 32, 34)[:br, : bc // 32].any()
+    # a constant 1.0 (code 0x38) under distinct scales reads back as the scale of its cell
+    ones = np.full((out, inn), 0x38, np.uint8)
+    grid = (120 + np.arange(9, dtype=np.uint8)).reshape(3, 3)
+    rows = ref.q8_0_repack_rows(ref.q8_0_from_hf(ones, grid, ref.SRC_F8E4M3), out, inn // 32)
+    y = ref.q8_0_dequant_rows(rows, out, inn)
+    want = np.repeat(np.repeat(np.exp2(grid.astype(np.float64) - 127), br, axis=0), bc, axis=1)
+    assert np.allclose(y, want, rtol=2e-3, atol=0)
+
+
+def test_q8_0_from_bf16_and_f32_checkpoint():
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(22)
+    x = (rng.standard_normal((8, 96)) * 0.02).astype(np.float32)
+    bits = torch.from_numpy(x).bfloat16().view(torch.int16).numpy().view(np.uint16)
+    xb = torch.from_numpy(x).bfloat16().float().numpy()
+    assert np.array_equal(ref.q8_0_from_hf(bits, None, ref.SRC_BF16), _q8_0_blocks_numpy(xb))
+    g = ref.q8_0_from_hf(x, None, ref.SRC_F32)
+    assert np.array_equal(g, _q8_0_blocks_numpy(x))
+    # split rows = the same blocks, scales first (crates/v4flash-kernels/src/weights.rs:225-240)
+    assert np.array_equal(ref.q8_0_repack_rows(g, 8, 3), ref.q8_0_quantize_rows(x))
+    b3 = g.reshape(8, 3, 34)
+    manual = np.concatenate([b3[:, :, :2].reshape(8, -1), b3[:, :, 2:].reshape(8, -1)], axis=1)
+    assert np.array_equal(ref.q8_0_repack_rows(g, 8, 3), manual.reshape(-1))
+
+
+def test_q8_0_from_fp8_refuses_what_the_reference_refuses():
+    codes = np.zeros((64, 64), np.uint8)
+    with pytest.raises(ValueError):
+        ref.q8_0_from_hf(codes, None, ref.SRC_F8E4M3)              # fp8 without scales
+    with pytest.raises(ValueError):
+        ref.q8_0_from_hf(codes, np.full((3, 2), 127, np.uint8), ref.SRC_F8E4M3)  # 64 % 3 != 0
+
+
 def test_q8_0_activation_quantizer():
     rng = np.random.default_rng(6)
     x = rng.standard_normal(128).astype(np.float32)
