@@ -56,6 +56,7 @@ SIGNATURES = {
     "dsx_init": (_int, []),
     "dsx_router_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _f32, _u32, _u32, _u32, _u32]),
     "dsx_router_logits": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "dsx_router_logits_f16": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "dsx_q8k_quantize": (_int, [_vp, _vp, _vp, _u32]),
     "dsx_q8_0_quantize": (_int, [_vp, _vp, _vp, _vp, _u32]),
     "dsx_q8_0_quantize_rows": (_int, [_vp, _vp, _vp, _u32, _u32]),
@@ -82,6 +83,7 @@ SIGNATURES = {
     "dsx_moe_layer_set_tuning": (_int, [_vp, _u32, _u32, _u32]),
     "dsx_moe_layer_workspace_bytes": (_sz, [_vp, _u32]),
     "dsx_moe_block_forward": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
+    "dsx_moe_block_forward_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
     "dsx_moe_layer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _sz, _vp, _vp, _vp, _vp]),
 }
 

@@ -517,17 +517,32 @@ int dsx_moe_reduce_partials(dsx_stream_t stream, float *out, const float *partia
     return reduce_impl(S(stream), out, partials, selected, nullptr, n_used, n_rows, b);
 }
 
-int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w, const float *x,
-                      uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
+extern "C++" {
+namespace {
+template <typename WT>
+int router_logits_impl(dsx_stream_t stream, float *logits, const WT *router_w, const float *x,
+                       uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
     if (n_tokens == 0) return DSX_OK;
     if (!logits || !router_w || !x) return fail(DSX_ERR_INVALID_ARG, "router_logits: null pointer");
     if (n_expert == 0 || hidden == 0) return fail(DSX_ERR_INVALID_ARG, "router_logits: n_expert=%u hidden=%u", n_expert, hidden);
     if (!aligned(router_w, 16) || !aligned(x, 16))
         return fail(DSX_ERR_SHAPE, "router_logits: router_w and x must be 16-byte aligned");
-    hipLaunchKernelGGL(k_router_logits<false>, dim3(n_expert), dim3(256), 0, S(stream), logits,
+    hipLaunchKernelGGL((k_router_logits<false, WT>), dim3(n_expert), dim3(256), 0, S(stream), logits,
                        (float *)nullptr, router_w, x, (const float *)nullptr, 0.0f, n_expert, hidden,
                        n_tokens);
     return launched("router_logits");
+}
+}  // namespace
+}  // extern "C++"
+
+int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w, const float *x,
+                      uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
+    return router_logits_impl(stream, logits, router_w, x, n_expert, hidden, n_tokens);
+}
+
+int dsx_router_logits_f16(dsx_stream_t stream, float *logits, const uint16_t *router_w,
+                          const float *x, uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
+    return router_logits_impl(stream, logits, (const __half *)router_w, x, n_expert, hidden, n_tokens);
 }
 
 // ---- element-wise -----------------------------------------------------------------------

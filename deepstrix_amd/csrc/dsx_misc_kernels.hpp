@@ -624,10 +624,22 @@ __device__ __forceinline__ void block_sum_256_multi(float (&v)[N], float *red, u
 // dot product are accumulated in the same sweep and reduced together, so the kernel has one
 // round of loads on its critical path; the workgroups whose index is a token id then write
 // that token's normalized row.
-template <bool NORM>
+// Router weights are f32 or f16 (the engine keeps ffn_gate_inp in f16,
+// crates/v4flash-kernels/src/f16.rs:37-45); products and sums are f32 either way.
+__device__ __forceinline__ float4 router_w4(const float *p) { return *(const float4 *)p; }
+__device__ __forceinline__ float4 router_w4(const __half *p) {
+    const uint2 v = *(const uint2 *)p;
+    const __half2 a = *(const __half2 *)&v.x, b = *(const __half2 *)&v.y;
+    const float2 fa = __half22float2(a), fb = __half22float2(b);
+    return make_float4(fa.x, fa.y, fb.x, fb.y);
+}
+__device__ __forceinline__ float router_w1(const float *p) { return *p; }
+__device__ __forceinline__ float router_w1(const __half *p) { return __half2float(*p); }
+
+template <bool NORM, typename WT>
 __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logits,
                                                        float *__restrict__ xn,
-                                                       const float *__restrict__ w,
+                                                       const WT *__restrict__ w,
                                                        const float *__restrict__ x,
                                                        const float *__restrict__ norm_w, float eps,
                                                        uint32_t n_expert, uint32_t hidden,
@@ -635,8 +647,8 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
     __shared__ float s_red[4 * 2 * kRlTokens];
     const uint32_t tid = threadIdx.x;
     const uint32_t e = blockIdx.x;
-    const float *wr = w + (uint64_t)e * hidden;
-    // float4 loads need 16-byte aligned rows; otherwise everything goes one element at a time
+    const WT *wr = w + (uint64_t)e * hidden;
+    // vector loads need aligned rows; otherwise everything goes one element at a time
     const uint32_t n4 = (hidden % 4u == 0u) ? hidden / 4u : 0u;
     for (uint32_t t0 = 0; t0 < n_tokens; t0 += kRlTokens) {
         const uint32_t nt = min((uint32_t)kRlTokens, n_tokens - t0);
@@ -649,7 +661,7 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
         }
 #pragma unroll 4
         for (uint32_t i = tid; i < n4; i += 256u) {
-            const float4 wv = *(const float4 *)(wr + 4u * i);
+            const float4 wv = router_w4(wr + 4u * i);
             float4 nw = {1.f, 1.f, 1.f, 1.f};
             if (NORM) nw = *(const float4 *)(norm_w + 4u * i);
 #pragma unroll
@@ -672,7 +684,7 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
             }
         }
         for (uint32_t i = 4u * n4 + tid; i < hidden; i += 256u) {
-            const float wv = wr[i];
+            const float wv = router_w1(wr + i);
 #pragma unroll
             for (int j = 0; j < kRlTokens; j++) {
                 if ((uint32_t)j < nt) {

@@ -47,10 +47,16 @@ def router_topk(selected, weights, logits, bias, n_expert, n_used, scale, eps, b
 
 
 def router_logits(logits, router_w, x, n_expert, hidden, n_tokens):
-    """crates/v4flash-kernels/kernels/laguna_ops.hip:57-60 (f32 W . x)"""
+    """crates/v4flash-kernels/kernels/laguna_ops.hip:57-60 (f32 W . x); f16 router weights as
+    crates/v4flash-kernels/src/f16.rs:37-45 keeps them take the f16 entry point."""
     capi.init()
-    check(lib().dsx_router_logits(_stream(), _p(logits), _p(router_w), _p(x), n_expert, hidden,
-                                  n_tokens))
+    if router_w.dtype == torch.float16:
+        fn = lib().dsx_router_logits_f16
+    elif router_w.dtype == torch.float32:
+        fn = lib().dsx_router_logits
+    else:
+        raise TypeError(f"router_w must be float32 or float16, got {router_w.dtype}")
+    check(fn(_stream(), _p(logits), _p(router_w), _p(x), n_expert, hidden, n_tokens))
 
 
 def q8k_quantize(out, x, n_blocks):

@@ -112,7 +112,13 @@ class MoeLayer:
         w = self.w
         if w.norm_w is None or w.router_w is None:
             raise ValueError("block() needs norm_w and router_w")
-        check(lib().dsx_moe_block_forward(
+        if w.router_w.dtype == torch.float16:
+            fn = lib().dsx_moe_block_forward_f16
+        elif w.router_w.dtype == torch.float32:
+            fn = lib().dsx_moe_block_forward
+        else:
+            raise TypeError(f"router_w must be float32 or float16, got {w.router_w.dtype}")
+        check(fn(
             self._h, torch.cuda.current_stream().cuda_stream, h.data_ptr(), w.norm_w.data_ptr(),
             w.norm_eps, w.router_w.data_ptr(), T, self.workspace.data_ptr(), self.workspace_bytes))
         return h

@@ -83,6 +83,11 @@ int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, cons
  * crates/v4flash-kernels/src/het/forward_prefill.rs:8974-9015). */
 int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w, const float *x,
                       uint32_t n_expert, uint32_t hidden, uint32_t n_tokens);
+/* The same with the router weights in f16, as the engine keeps ffn_gate_inp
+ * (F16Matvec::matvec_batched_router, crates/v4flash-kernels/src/f16.rs:37-45; call site
+ * crates/v4flash-kernels/src/het/forward_prefill.rs:9008-9016): f32 products and sums. */
+int dsx_router_logits_f16(dsx_stream_t stream, float *logits, const uint16_t *router_w,
+                          const float *x, uint32_t n_expert, uint32_t hidden, uint32_t n_tokens);
 
 /* ---- activation quantizers ------------------------------------------------
  * Q8KQuantize::launch (crates/v4flash-kernels/src/q8_k.rs:33-104). */
@@ -263,6 +268,10 @@ int dsx_moe_layer_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
 int dsx_moe_block_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *h, const float *norm_w,
                           float eps, const float *router_w, uint32_t n_tokens, void *workspace,
                           size_t workspace_bytes);
+/* The same block with router_w in f16 [n_expert, hidden] (see dsx_router_logits_f16). */
+int dsx_moe_block_forward_f16(dsx_moe_layer *layer, dsx_stream_t stream, float *h,
+                              const float *norm_w, float eps, const uint16_t *router_w,
+                              uint32_t n_tokens, void *workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -48,6 +48,38 @@ def test_router_logits_operator():
         np.testing.assert_allclose(out.cpu().numpy(), ref.router_logits(W, x), atol=3e-5)
 
 
+def test_router_logits_operator_f16_weights():
+    """The engine keeps the router matrix in f16 (crates/v4flash-kernels/src/f16.rs:37-45):
+    products and sums stay f32, so the result equals the f32 matvec over the widened weights."""
+    rng = np.random.default_rng(1)
+    for T, E, hidden in [(1, 384, 5120), (5, 256, 7168), (9, 16, 520), (3, 7, 30), (2, 5, 1026)]:
+        W16 = rng.normal(0, 0.02, (E, hidden)).astype(np.float16)
+        x = rng.normal(0, 1, (T, hidden)).astype(np.float32)
+        out = torch.zeros((T, E), dtype=torch.float32, device="cuda")
+        dispatch.router_logits(out, torch.from_numpy(W16).cuda(), torch.from_numpy(x).cuda(), E, hidden, T)
+        np.testing.assert_allclose(out.cpu().numpy(), ref.router_logits(W16.astype(np.float32), x),
+                                   atol=3e-5)
+    with pytest.raises(TypeError):
+        dispatch.router_logits(out, torch.zeros((E, hidden), dtype=torch.bfloat16, device="cuda"),
+                               torch.from_numpy(x).cuda(), E, hidden, T)
+
+
+@pytest.mark.parametrize("T", [1, 3, 130])
+def test_block_with_f16_router_weights_equals_block_with_the_widened_weights(T):
+    s = H.Shape(1024, 512, 16, 4, router_mode=1, n_group=4, topk_group=2, route_scale=2.5,
+                bias_sigma=0.01, clamp=10.0, seed=103)
+    dw = H.device_weights(s, block=True)
+    w16 = dw.router_w.to(torch.float16)
+    h, _, _ = H.host_inputs(s, T)
+    a = torch.from_numpy(h).cuda()
+    b = a.clone()
+    dw.router_w = w16.float()
+    MoeLayer(dw, T).block(a)
+    dw.router_w = w16
+    MoeLayer(dw, T).block(b)
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("T", [1, 2, 4, 6, 130])
 def test_block_matches_oracle(T):
     """decode path (residual fused into `down`), by-expert path and GEMM path."""
