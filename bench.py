@@ -285,6 +285,20 @@ def main():
     gu_avg_us = float(gu_ms.mean() * 1e3)
     achieved = GATE_UP_BYTES / (gu_avg_us * 1e-6) / 1e9
 
+    # what the bracket itself costs: the same pair of events around a one-workgroup kernel
+    # (a 16-byte add, about a microsecond of kernel time in a kernel trace)
+    from deepstrix_amd import dispatch
+    tiny_a = torch.zeros(4, dtype=torch.float32, device="cuda")
+    tiny_b = torch.ones(4, dtype=torch.float32, device="cuda")
+    tiny = [(hip.event(), hip.event()) for _ in range(64)]
+    for j, (a, b) in enumerate(tiny):
+        step(W + j % K)
+        hip.l.hipEventRecord(a, stream)
+        dispatch.vec_add_inplace(tiny_a, tiny_b, 4)
+        hip.l.hipEventRecord(b, stream)
+    torch.cuda.synchronize()
+    tiny_us = float(np.median([hip.elapsed_ms(a, b) for a, b in tiny]) * 1e3)
+
     # a copy of known size, so that byte counters collected over this run can be scaled
     from deepstrix_amd import synth
     c_src = torch.empty(COPY_BYTES, dtype=torch.uint8, device="cuda").random_(0, 255)
@@ -296,6 +310,7 @@ def main():
 
     # other token counts of the same config (informative)
     extra = {"gate_up_us_p50": float(np.median(gu_ms) * 1e3),
+             "event_bracket_of_one_workgroup_kernel_us": tiny_us,
              "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
              "layer_GBps_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9,
              "layer_frac_of_hbm_peak_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}

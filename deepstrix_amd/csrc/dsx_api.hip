@@ -48,9 +48,17 @@ void allow_lds(K kernel) {
                               160 * 1024 - 16 * 1024);
 }
 
-std::once_flag g_attr_once;
+// Function attributes belong to a device: raised once per device, with that device current.
+constexpr int kMaxDevices = 64;
+std::mutex g_attr_mutex;
+bool g_attr_done[kMaxDevices] = {};
 void raise_lds_limits() {
-    std::call_once(g_attr_once, [] {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(g_attr_mutex);
+    if (g_attr_done[dev]) return;
+    g_attr_done[dev] = true;
+    {
         allow_lds(k_mxfp4_gate_up<1, false, false, false>);
         allow_lds(k_mxfp4_gate_up<1, false, true, true>);
         allow_lds(k_mxfp4_gate_up<1, true, false, false>);
@@ -76,7 +84,7 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_down_by_expert<8, true>);
         allow_lds(k_mxfp4_down_by_expert<16, true>);
         q8_0_raise_lds_limits();
-    });
+    }
 }
 
 constexpr size_t kLdsBudget = 140 * 1024;  // dynamic LDS a workgroup may ask for
