@@ -97,26 +97,33 @@ int pick_nt(uint32_t chunk) {
     return 16;
 }
 
+// max_wi work items, p.n_sub workgroups along grid.y for each
 template <int NT>
 static void launch_gate_up_be(hipStream_t st, const GateUpParams &p, uint32_t max_wi, size_t lds,
                               bool staged) {
+    const dim3 grid(p.n_rows / 16, max_wi * p.n_sub);
     if (staged)
-        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, true, false>), dim3(p.n_rows / 16, max_wi),
-                           dim3(kGuWaves * 64), lds, st, p);
+        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, true, false>), grid, dim3(kGuWaves * 64), lds, st, p);
     else
-        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, false, false>), dim3(p.n_rows / 16, max_wi),
-                           dim3(kGuWaves * 64), lds, st, p);
+        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, false, false>), grid, dim3(kGuWaves * 64), lds, st, p);
 }
 
 template <int NT>
 static void launch_down_be(hipStream_t st, const DownByExpertParams &p, uint32_t max_wi, size_t lds,
                            bool staged) {
+    const dim3 grid(p.n_rows / 16, max_wi * p.n_sub);
     if (staged)
-        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, true>), dim3(p.n_rows / 16, max_wi),
-                           dim3(kDownBeWaves * 64), lds, st, p);
+        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, true>), grid, dim3(kDownBeWaves * 64), lds, st, p);
     else
-        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, false>), dim3(p.n_rows / 16, max_wi),
-                           dim3(kDownBeWaves * 64), lds, st, p);
+        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, false>), grid, dim3(kDownBeWaves * 64), lds, st, p);
+}
+
+// Columns per workgroup for a work item of `chunk` members: the largest power of two (at most
+// `cap`) whose activation tiles fit LDS; a larger chunk is served by several workgroups per item.
+static int fit_nt(uint32_t chunk, uint32_t n_blocks, int cap) {
+    int nt = std::min(pick_nt(chunk), cap);
+    while (nt > 1 && (size_t)n_blocks * 512 * nt + (size_t)n_blocks * nt * 4 > kLdsBudget) nt /= 2;
+    return nt;
 }
 
 
@@ -392,7 +399,8 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: null pointer");
     if (max_work_items > 65535)
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: max_work_items=%u", max_work_items);
-    if (chunk == 0 || chunk > 16) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: chunk=%u", chunk);
+    if (chunk == 0 || chunk > 64)
+        return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: chunk=%u not in 1..64", chunk);
     if (dtype == DSX_FMT_Q8_0)
         return q8_0_gate_up_by_expert(S(stream), mid, gate, up, xq, ew, group_count, group_offset,
                                       expert_members, work_items, n_work_items, max_work_items,
@@ -405,12 +413,15 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     if (n_blocks == 0) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: n_blocks=0");
     if (gbpe % 8 || ubpe % 8 || !aligned(gate, 8) || !aligned(up, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: weights must be 8-byte aligned, xq 4-byte");
-    const int nt = pick_nt(chunk);
+    const int nt = fit_nt(chunk, n_blocks, 8);
     const size_t lds = (size_t)n_blocks * 512 * nt + (size_t)n_blocks * nt * 4;
-    if (lds > kLdsBudget || nt > 8)
-        return fail(DSX_ERR_UNSUPPORTED,
-                    "moe_gate_up_chunked_rows: chunk=%u x n_blocks=%u needs %zu B of LDS", chunk,
+    if (lds > kLdsBudget)
+        return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows: n_blocks=%u needs %zu B of LDS",
                     n_blocks, lds);
+    const uint32_t n_sub = (chunk + (uint32_t)nt - 1u) / (uint32_t)nt;
+    if ((uint64_t)max_work_items * n_sub > 65535u)
+        return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: %u work items x %u sub-chunks exceed the grid",
+                    max_work_items, n_sub);
     raise_lds_limits();
     GateUpParams p{};
     p.mid = mid; p.gate = gate; p.up = up; p.xq = xq; p.ew = ew;
@@ -420,6 +431,7 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     p.n_rows = n_rows; p.n_blocks = n_blocks;
     p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
     p.sh_gate = sh_gate; p.sh_up = sh_up; p.sh_clamp = sh_clamp; p.n_expert = n_expert; p.n_tokens = n_tokens;
+    p.n_sub = n_sub;
     hipStream_t st = S(stream);
     switch (nt) {
         case 1: launch_gate_up_be<1>(st, p, max_work_items, lds, staged); break;
@@ -456,7 +468,8 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
         return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: null pointer");
     if (max_work_items > 65535)
         return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: max_work_items=%u", max_work_items);
-    if (chunk == 0 || chunk > 16) return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: chunk=%u", chunk);
+    if (chunk == 0 || chunk > 64)
+        return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: chunk=%u not in 1..64", chunk);
     if (dtype == DSX_FMT_Q8_0)
         return q8_0_down_by_expert(S(stream), partials, down, xq, group_count, group_offset,
                                    expert_members, work_items, n_work_items, max_work_items, dbpe,
@@ -472,11 +485,15 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: xq_slot_stride=%u", xq_slot_stride);
     if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: weights must be 8-byte aligned, xq 4-byte");
-    const int nt = pick_nt(chunk);
+    const int nt = fit_nt(chunk, n_blocks_in, 16);
     const size_t lds = (size_t)n_blocks_in * 512 * nt + (size_t)n_blocks_in * nt * 4;
     if (lds > kLdsBudget)
-        return fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert: chunk=%u x n_blocks_in=%u needs %zu B of LDS",
-                    chunk, n_blocks_in, lds);
+        return fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert: n_blocks_in=%u needs %zu B of LDS",
+                    n_blocks_in, lds);
+    const uint32_t n_sub = (chunk + (uint32_t)nt - 1u) / (uint32_t)nt;
+    if ((uint64_t)max_work_items * n_sub > 65535u)
+        return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: %u work items x %u sub-chunks exceed the grid",
+                    max_work_items, n_sub);
     raise_lds_limits();
     DownByExpertParams p{};
     p.partials = partials; p.down = down; p.xq = xq;
@@ -485,6 +502,7 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
     p.sh_down = sh_down; p.n_expert = n_expert; p.n_tokens = n_tokens;
+    p.n_sub = n_sub;
     hipStream_t st = S(stream);
     switch (nt) {
         case 1: launch_down_be<1>(st, p, max_work_items, lds, staged); break;

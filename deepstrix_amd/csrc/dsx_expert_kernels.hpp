@@ -112,6 +112,9 @@ struct GateUpParams {
     // by-expert with the extra expert (index n_expert, slot n_used; its rows follow the
     // n_tokens * n_used routed ones): sh_gate / sh_up / sh_clamp above, and
     uint32_t n_expert, n_tokens;
+    // by-expert: a work item of `chunk` members is served by n_sub workgroups along grid.y,
+    // NT columns each (0 is read as 1)
+    uint32_t n_sub;
 };
 
 // LDS: [n_blocks] tiles of 512 * NT bytes | yd[n_blocks * NT] floats
@@ -129,7 +132,9 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t row0 = blockIdx.x * 16u;
-    const uint32_t item = blockIdx.y;
+    const uint32_t n_sub = (BY_EXPERT && p.n_sub > 1u) ? p.n_sub : 1u;
+    const uint32_t item = blockIdx.y / n_sub;
+    const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;  // first member served here
     // decode from a staged row that one pass of the workgroup covers: loaded before the weights
     const bool early = !BY_EXPERT && STAGED && NT == 1 && p.n_blocks * 32u <= 4u * kGuWaves * 64u;
     uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {};
@@ -142,10 +147,10 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     if (BY_EXPERT) {
         if ((int)item >= *p.n_work_items) return;  // uniform: grid is an upper bound
         const uint32_t wi = (uint32_t)p.work_items[item];
-        const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
+        const uint32_t e = wi >> 16, start = (wi & 0xFFFFu) + col_off;
         const uint32_t total = (uint32_t)p.group_count[e];
-        cnt = min(p.chunk, total - start);
-        if (cnt > (uint32_t)NT) cnt = NT;
+        if (start >= total) return;  // uniform: this sub-chunk of the item has no members
+        cnt = min(min(p.chunk - col_off, (uint32_t)NT), total - start);
         const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
         const bool extra = p.sh_gate != nullptr && e >= p.n_expert;
         if (tid < cnt) {
@@ -484,6 +489,7 @@ struct DownByExpertParams {
     uint32_t xq_slot_stride, n_used, chunk, n_rows, n_blocks_in;
     const uint8_t *sh_down;  // the extra expert (index n_expert, slot n_used), or null
     uint32_t n_expert, n_tokens;
+    uint32_t n_sub;  // workgroups along grid.y per work item, NT columns each (0 is read as 1)
 };
 
 // LDS: [n_blocks_in] tiles of 512 * NT bytes | yd[n_blocks_in * NT]
@@ -500,12 +506,15 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t row0 = blockIdx.x * 16u;
-    const uint32_t item = blockIdx.y;
+    const uint32_t n_sub = p.n_sub > 1u ? p.n_sub : 1u;
+    const uint32_t item = blockIdx.y / n_sub;
+    const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;
     if ((int)item >= *p.n_work_items) return;
     const uint32_t wi = (uint32_t)p.work_items[item];
-    const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
-    uint32_t cnt = min(p.chunk, (uint32_t)p.group_count[e] - start);
-    if (cnt > (uint32_t)NT) cnt = NT;
+    const uint32_t e = wi >> 16, start = (wi & 0xFFFFu) + col_off;
+    const uint32_t total = (uint32_t)p.group_count[e];
+    if (start >= total) return;  // uniform: this sub-chunk of the item has no members
+    const uint32_t cnt = min(min(p.chunk - col_off, (uint32_t)NT), total - start);
     const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
     const bool extra = p.sh_down != nullptr && e >= p.n_expert;
     if (tid < cnt) {

@@ -44,6 +44,8 @@ struct Q8Params {
     float clamp, sh_clamp;
     // by-expert with the extra expert (index n_expert, slot n_used; rows after the routed ones)
     uint32_t n_expert, n_tokens;
+    // by-expert: workgroups along grid.y per work item, NT columns each (0 is read as 1)
+    uint32_t n_sub;
 };
 
 // The lane's share of `row . x[c]` for NT columns, over all of its blocks.
@@ -106,7 +108,9 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_gate_up(const Q8Params p
     __shared__ uint32_t s_dest[NT];
     __shared__ float s_ew[NT];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y;
+    const uint32_t n_sub = (BY_EXPERT && p.n_sub > 1u) ? p.n_sub : 1u;
+    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y / n_sub;
+    const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;  // first member served here
     const uint32_t row_bytes = q8_0_act_row_bytes(p.n_blocks);
     const uint8_t *g_e, *u_e;
     uint32_t cnt = 1;
@@ -114,8 +118,10 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_gate_up(const Q8Params p
     if (BY_EXPERT) {
         if ((int)item >= *p.n_work_items) return;
         const uint32_t wi = (uint32_t)p.work_items[item];
-        const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
-        cnt = min(min(p.chunk, (uint32_t)NT), (uint32_t)p.group_count[e] - start);
+        const uint32_t e = wi >> 16, start = (wi & 0xFFFFu) + col_off;
+        const uint32_t total = (uint32_t)p.group_count[e];
+        if (start >= total) return;  // uniform: this sub-chunk of the item has no members
+        cnt = min(min(p.chunk - col_off, (uint32_t)NT), total - start);
         const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
         if (tid < cnt) {
             const uint32_t m = (uint32_t)p.members[mbase + tid];
@@ -217,12 +223,16 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_by_expert(const Q8P
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];
     __shared__ uint32_t s_dest[NT];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y;
+    const uint32_t n_sub = p.n_sub > 1u ? p.n_sub : 1u;
+    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y / n_sub;
+    const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;
     const uint32_t row_bytes = q8_0_act_row_bytes(p.n_blocks);
     if ((int)item >= *p.n_work_items) return;
     const uint32_t wi = (uint32_t)p.work_items[item];
-    const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
-    const uint32_t cnt = min(min(p.chunk, (uint32_t)NT), (uint32_t)p.group_count[e] - start);
+    const uint32_t e = wi >> 16, start = (wi & 0xFFFFu) + col_off;
+    const uint32_t total = (uint32_t)p.group_count[e];
+    if (start >= total) return;  // uniform: this sub-chunk of the item has no members
+    const uint32_t cnt = min(min(p.chunk - col_off, (uint32_t)NT), total - start);
     const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
     if (tid < cnt) {
         const uint32_t m = (uint32_t)p.members[mbase + tid];
@@ -281,6 +291,13 @@ inline int q8_0_check(const char *what, uint32_t n_rows, uint32_t n_blocks, cons
 }
 
 inline int q8_0_pick_nt(uint32_t chunk) { return chunk <= 1 ? 1 : chunk <= 2 ? 2 : chunk <= 4 ? 4 : 8; }
+// Columns per workgroup for a work item of `chunk` members: as many as LDS stages (at most 8);
+// a larger chunk is served by several workgroups per item.
+inline int q8_0_fit_nt(uint32_t chunk, uint32_t n_blocks) {
+    int nt = q8_0_pick_nt(chunk);
+    while (nt > 1 && (size_t)nt * q8_0_act_row_bytes(n_blocks) > kQ8LdsBudget) nt /= 2;
+    return nt;
+}
 
 inline int q8_0_gate_up_decode(hipStream_t st, float *mid, const uint8_t *gate, const uint8_t *up,
                                const uint8_t *xq, const float *ew, const int32_t *selected,
@@ -327,8 +344,10 @@ inline int q8_0_gate_up_by_expert(hipStream_t st, float *mid, const uint8_t *gat
                                   uint32_t chunk, float clamp, uint32_t n_rows, uint32_t n_blocks,
                                   const uint8_t *sh_gate = nullptr, const uint8_t *sh_up = nullptr,
                                   float sh_clamp = 0.0f, uint32_t n_expert = 0, uint32_t n_tokens = 0) {
-    if (chunk > 8) return q8_0_fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows", "Q8_0 takes chunk <= 8");
-    const int nt = q8_0_pick_nt(chunk);
+    const int nt = q8_0_fit_nt(chunk, n_blocks);
+    const uint32_t n_sub = (chunk + (uint32_t)nt - 1u) / (uint32_t)nt;
+    if ((uint64_t)max_wi * n_sub > 65535u)
+        return q8_0_fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows", "work items x sub-chunks exceed the grid");
     int rc = q8_0_check("moe_gate_up_chunked_rows", n_rows, n_blocks, gate, up, gbpe, ubpe, xq,
                         q8_0_act_row_bytes(n_blocks), (uint32_t)nt);
     if (rc) return rc;
@@ -339,7 +358,8 @@ inline int q8_0_gate_up_by_expert(hipStream_t st, float *mid, const uint8_t *gat
     p.x_stride = q8_0_act_row_bytes(n_blocks); p.n_used = n_used; p.chunk = chunk; p.n_rows = n_rows;
     p.n_blocks = n_blocks; p.clamp = clamp;
     p.sh_w0 = sh_gate; p.sh_w1 = sh_up; p.sh_clamp = sh_clamp; p.n_expert = n_expert; p.n_tokens = n_tokens;
-    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi), block(kQ8Waves * 64);
+    p.n_sub = n_sub;
+    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi * n_sub), block(kQ8Waves * 64);
     const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks);
     switch (nt) {
         case 1: hipLaunchKernelGGL((k_q8_0_gate_up<1, true>), grid, block, lds, st, p); break;
@@ -358,8 +378,10 @@ inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *d
                                uint32_t xq_slot_stride, uint32_t n_used, uint32_t chunk,
                                uint32_t n_rows, uint32_t n_blocks_in, const uint8_t *sh_down = nullptr,
                                uint32_t n_expert = 0, uint32_t n_tokens = 0) {
-    if (chunk > 8) return q8_0_fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert", "Q8_0 takes chunk <= 8");
-    const int nt = q8_0_pick_nt(chunk);
+    const int nt = q8_0_fit_nt(chunk, n_blocks_in);
+    const uint32_t n_sub = (chunk + (uint32_t)nt - 1u) / (uint32_t)nt;
+    if ((uint64_t)max_wi * n_sub > 65535u)
+        return q8_0_fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert", "work items x sub-chunks exceed the grid");
     int rc = q8_0_check("moe_down_by_expert", n_rows, n_blocks_in, down, nullptr, dbpe, 0, xq,
                         xq_slot_stride, (uint32_t)nt);
     if (rc) return rc;
@@ -370,7 +392,8 @@ inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *d
     p.x_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk; p.n_rows = n_rows;
     p.n_blocks = n_blocks_in;
     p.sh_w0 = sh_down; p.n_expert = n_expert; p.n_tokens = n_tokens;
-    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi), block(kQ8Waves * 64);
+    p.n_sub = n_sub;
+    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi * n_sub), block(kQ8Waves * 64);
     const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks_in);
     switch (nt) {
         case 1: hipLaunchKernelGGL(k_q8_0_down_by_expert<1>, grid, block, lds, st, p); break;

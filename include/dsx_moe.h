@@ -126,7 +126,8 @@ int dsx_moe_down_batched(dsx_stream_t stream, int dtype, float *out, const uint8
  * n_work_items[1].  Unlike the reference's atomic builder the order is
  * deterministic and the member table is compacted (no max_per_expert).
  * selected entries outside [0, n_expert) are skipped.  b, n_used, n_expert <
- * 65536; chunk in [1, 64] (the by-expert entry points below take chunk <= 16). */
+ * 65536; chunk in [1, 64] (the reference executor uses 32,
+ * crates/v4flash-kernels/src/het/remote_experts.rs:77). */
 int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,
                         int32_t *expert_members, int32_t *work_items, int32_t *n_work_items,
                         const int32_t *selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
@@ -134,7 +135,9 @@ int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *grou
 /* dispatch::moe_gate_up_chunked_rows (crates/v4flash-kernels/src/het/dispatch.rs:534-570):
  * mid[b, n_used, n_rows]; xq is [b, n_blocks*292]; ew is [b, n_used].
  * max_work_items bounds the grid (dispatch::moe_wi_upper_bound, :450-454); the
- * device-side count is read by the kernel. */
+ * device-side count is read by the kernel.  chunk (1..64) is the one the work items
+ * were built with; an item wider than the columns one workgroup stages is served by
+ * several workgroups. */
 int dsx_moe_gate_up_chunked_rows(dsx_stream_t stream, int dtype, float *mid, const uint8_t *gate,
                                  const uint8_t *up, const uint8_t *xq, const float *ew,
                                  const int32_t *group_count, const int32_t *group_offset,

@@ -188,7 +188,9 @@ def test_group_build_matches_oracle(T, E, k, chunk):
     assert int(gc.sum()) == int((sel >= 0).sum())
 
 
-@pytest.mark.parametrize("T,chunk", [(5, 4), (9, 2), (3, 1), (12, 8)])
+# chunk 32 is the reference executor's CHUNK_SIZE (crates/v4flash-kernels/src/het/remote_experts.rs:77):
+# a work item wider than one workgroup's columns is served by several workgroups
+@pytest.mark.parametrize("T,chunk", [(5, 4), (9, 2), (3, 1), (12, 8), (45, 32), (70, 64), (21, 20)])
 def test_by_expert_chain_matches_oracle(T, chunk):
     s, w = small_case(hidden=768, inter=256, E=8, k=3, seed=21)
     gb = synth.matrix_bytes(FMT_MXFP4, s.inter, s.hidden)

@@ -84,7 +84,7 @@ def test_q8_0_one_hot_activation_reads_single_weights():
             np.testing.assert_allclose(mid.cpu().numpy()[0], g / (1 + np.exp(-g)) * u, rtol=3e-6, atol=1e-30)
 
 
-@pytest.mark.parametrize("T,chunk", [(5, 4), (9, 2), (3, 1), (20, 8)])
+@pytest.mark.parametrize("T,chunk", [(5, 4), (9, 2), (3, 1), (20, 8), (45, 32), (21, 20)])
 def test_q8_0_by_expert_chain_matches_oracle(T, chunk):
     s, w = q8_case(hidden=384, inter=128, E=5, k=2, seed=33)
     gb = synth.matrix_bytes(FMT_Q8_0, s.inter, s.hidden)
