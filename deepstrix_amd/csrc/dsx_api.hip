@@ -209,6 +209,22 @@ int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, cons
     return launched("router_topk");
 }
 
+int dsx_router_hash_select(dsx_stream_t stream, int32_t *selected, float *weights,
+                           const float *logits, const int32_t *tid2eid, const int32_t *token_ids,
+                           uint32_t n_expert, uint32_t n_used, uint32_t vocab, float scale,
+                           float eps, uint32_t b) {
+    if (b == 0) return DSX_OK;
+    if (!selected || !weights || !logits || !tid2eid || !token_ids)
+        return fail(DSX_ERR_INVALID_ARG, "router_hash_select: null pointer");
+    if (n_expert == 0 || vocab == 0)
+        return fail(DSX_ERR_INVALID_ARG, "router_hash_select: n_expert=%u vocab=%u", n_expert, vocab);
+    if (n_used == 0 || n_used > DSX_MAX_USED)
+        return fail(DSX_ERR_INVALID_ARG, "router_hash_select: n_used=%u not in 1..%d", n_used, DSX_MAX_USED);
+    hipLaunchKernelGGL(k_router_hash_select, dim3((b + 255) / 256), dim3(256), 0, S(stream), selected,
+                       weights, logits, tid2eid, token_ids, n_expert, n_used, vocab, scale, eps, b);
+    return launched("router_hash_select");
+}
+
 // ---- quantizers -----------------------------------------------------------------------
 int dsx_q8k_quantize(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t n_blocks) {
     if (n_blocks == 0) return DSX_OK;

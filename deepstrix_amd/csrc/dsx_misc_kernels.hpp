@@ -217,6 +217,37 @@ __global__ __launch_bounds__(kRouterThreads) void k_router_topk(
                 topk_group);
 }
 
+// Hash routing of the bootstrap layers: the picks of a token are row `token id` of
+// tid2eid[vocab, n_used]; weights = sqrt(softplus(logit)) / max(sum, eps) * scale with the sum
+// in slot order.  One thread per token (n_used <= 16).  An id out of range leaves an empty
+// slot (-1, weight 0).  crates/v4flash-kernels/src/routing.rs:21-44.
+__global__ __launch_bounds__(256) void k_router_hash_select(
+    int32_t *__restrict__ selected, float *__restrict__ weights, const float *__restrict__ logits,
+    const int32_t *__restrict__ tid2eid, const int32_t *__restrict__ token_ids, uint32_t n_expert,
+    uint32_t n_used, uint32_t vocab, float scale, float eps, uint32_t n_tokens) {
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= n_tokens) return;
+    const int tok = token_ids[t];
+    const bool tok_ok = tok >= 0 && (uint32_t)tok < vocab;
+    const float *lg = logits + (uint64_t)t * n_expert;
+    float w[DSX_MAX_USED_K];
+    float sum = 0.0f;
+#pragma unroll
+    for (uint32_t i = 0; i < DSX_MAX_USED_K; i++) {
+        if (i < n_used) {
+            int e = tok_ok ? tid2eid[(uint64_t)tok * n_used + i] : -1;
+            if (e < 0 || (uint32_t)e >= n_expert) e = -1;
+            selected[(uint64_t)t * n_used + i] = e;
+            w[i] = (e >= 0) ? sqrtf(softplus_stable(lg[e])) : 0.0f;
+            sum += w[i];
+        }
+    }
+    if (sum < eps) sum = eps;
+#pragma unroll
+    for (uint32_t i = 0; i < DSX_MAX_USED_K; i++)
+        if (i < n_used) weights[(uint64_t)t * n_used + i] = w[i] / sum * scale;
+}
+
 // Front of the layer in one launch: workgroups [0, n_tokens) route one token each (skipped
 // when routing is pinned), the rest quantize the activations into staged rows (one wave per
 // 256-element block) and clear the arrival counters of the fused mid quantization.

@@ -46,6 +46,15 @@ def router_topk(selected, weights, logits, bias, n_expert, n_used, scale, eps, b
                                 n_expert, n_used, scale, eps, b, mode, n_group, topk_group))
 
 
+def router_hash_select(selected, weights, logits, tid2eid, token_ids, scale=1.5, eps=6.103515625e-5):
+    """crates/v4flash-kernels/src/routing.rs:21-44, on the device (no logits readback)."""
+    capi.init()
+    b, n_expert = logits.shape
+    vocab, n_used = tid2eid.shape
+    check(lib().dsx_router_hash_select(_stream(), _p(selected), _p(weights), _p(logits), _p(tid2eid),
+                                       _p(token_ids), n_expert, n_used, vocab, scale, eps, b))
+
+
 def router_logits(logits, router_w, x, n_expert, hidden, n_tokens):
     """crates/v4flash-kernels/kernels/laguna_ops.hip:57-60 (f32 W . x); f16 router weights as
     crates/v4flash-kernels/src/f16.rs:37-45 keeps them take the f16 entry point."""

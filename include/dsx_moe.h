@@ -78,6 +78,18 @@ int dsx_router_topk(dsx_stream_t stream, int32_t *selected, float *weights, cons
                     const float *bias, uint32_t n_expert, uint32_t n_used, float scale, float eps,
                     uint32_t b, uint32_t mode, uint32_t n_group, uint32_t topk_group);
 
+/* hash_router_select (crates/v4flash-kernels/src/routing.rs:21-44; call sites
+ * het/forward_layer.rs:2253, het/forward_prefill.rs:9167): the picks of token t are row
+ * token_ids[t] of tid2eid[vocab, n_used]; weights[t,i] = sqrt(softplus(logits[t, pick])) /
+ * max(sum over the picks, eps) * scale.  The reference runs this on the host with n_used 6,
+ * eps 6.103515625e-5, scale 1.5 after reading the logits back; here everything stays on the
+ * device and feeds dsx_moe_layer_forward's selected_in / weights_in.  A token id outside
+ * [0, vocab) or an expert id outside [0, n_expert) gives an empty slot (-1, weight 0). */
+int dsx_router_hash_select(dsx_stream_t stream, int32_t *selected, float *weights,
+                           const float *logits, const int32_t *tid2eid, const int32_t *token_ids,
+                           uint32_t n_expert, uint32_t n_used, uint32_t vocab, float scale,
+                           float eps, uint32_t b);
+
 /* f32 router matvec: logits[t,e] = sum_k router_w[e,k] * x[t,k]
  * (crates/v4flash-kernels/kernels/laguna_ops.hip:57-60;
  * crates/v4flash-kernels/src/het/forward_prefill.rs:8974-9015). */

@@ -596,6 +596,32 @@ int dsx_ref_router_topk(int32_t *selected, float *weights, const float *logits,
     return 0;
 }
 
+/* K/src/routing.rs:21-44 (hash_router_select): the picks of token id `tok` are row `tok` of
+ * tid2eid[vocab, n_used]; weights sqrt(softplus(logit)) / max(sum, eps) * scale, the sum
+ * taken in slot order (the reference: n_used 6, eps 6.103515625e-5, scale 1.5).  A token id
+ * or an expert id out of range gives an empty slot (-1, weight 0) where the reference would
+ * index out of bounds. */
+void dsx_ref_router_hash_select(int32_t *selected, float *weights, const float *logits,
+                                const int32_t *tid2eid, const int32_t *token_ids, int n_expert,
+                                int n_used, int vocab, float scale, float eps, int n_tokens) {
+    for (int t = 0; t < n_tokens; t++) {
+        const int tok = token_ids[t];
+        const float *lg = logits + (size_t)t * n_expert;
+        int32_t *sel = selected + (size_t)t * n_used;
+        float *w = weights + (size_t)t * n_used;
+        float sum = 0.0f;
+        for (int i = 0; i < n_used; i++) {
+            int e = (tok >= 0 && tok < vocab) ? tid2eid[(size_t)tok * n_used + i] : -1;
+            if (e < 0 || e >= n_expert) e = -1;
+            sel[i] = e;
+            w[i] = (e >= 0) ? sqrtf(softplus_stable(lg[e])) : 0.0f;
+            sum += w[i];
+        }
+        if (sum < eps) sum = eps;
+        for (int i = 0; i < n_used; i++) w[i] = w[i] / sum * scale;
+    }
+}
+
 /* K/kernels/laguna_ops.hip:57-60 */
 void dsx_ref_router_logits(float *logits, const float *w, const float *x, int n_expert,
                            int hidden, int n_tokens) {

@@ -99,6 +99,7 @@ def _declare(l):
     l.dsx_ref_router_scores.restype = i32
     l.dsx_ref_router_scores.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32]
     l.dsx_ref_router_logits.argtypes = [vp, vp, vp, i32, i32, i32]
+    l.dsx_ref_router_hash_select.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, i32]
     l.dsx_ref_group_build.restype = i32
     l.dsx_ref_group_build.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32]
     l.dsx_ref_wi_upper_bound.restype = C.c_uint32
@@ -270,6 +271,21 @@ def router_topk(logits, bias, n_used, scale, eps, mode, n_group=1, topk_group=1)
                                    T, mode, n_group, topk_group)
     if rc != 0:
         raise ValueError(f"dsx_ref_router_topk rc={rc}")
+    return sel, w
+
+
+def router_hash_select(logits, tid2eid, token_ids, scale=1.5, eps=6.103515625e-5):
+    """crates/v4flash-kernels/src/routing.rs:21-44: picks from the token's row of tid2eid."""
+    logits = _c(logits, np.float32)
+    tid2eid = _c(tid2eid, np.int32)
+    token_ids = _c(token_ids, np.int32)
+    T, E = logits.shape
+    vocab, n_used = tid2eid.shape
+    assert token_ids.shape == (T,)
+    sel = np.empty((T, n_used), np.int32)
+    w = np.empty((T, n_used), np.float32)
+    lib().dsx_ref_router_hash_select(_p(sel), _p(w), _p(logits), _p(tid2eid), _p(token_ids), E,
+                                     n_used, vocab, scale, eps, T)
     return sel, w
 
 

@@ -231,6 +231,39 @@ def test_by_expert_chain_matches_oracle(T, chunk):
     assert H.max_rel(out.cpu().numpy(), out_ref) < 1e-5
 
 
+def test_hash_router_select_matches_oracle_and_feeds_the_layer():
+    # crates/v4flash-kernels/src/routing.rs:21-44, on the device
+    rng = np.random.default_rng(12)
+    E, k, vocab, T = 256, 6, 129, 300
+    tid2eid = np.stack([rng.choice(E, k, replace=False) for _ in range(vocab)]).astype(np.int32)
+    tid2eid[5, 1] = E          # out of range: empty slot
+    toks = rng.integers(0, vocab, T).astype(np.int32)
+    toks[:3] = [5, vocab, -2]
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[7] = -30.0
+    sel = torch.full((T, k), 99, dtype=torch.int32, device="cuda")
+    w = torch.full((T, k), np.nan, dtype=torch.float32, device="cuda")
+    dispatch.router_hash_select(sel, w, dev(logits), dev(tid2eid), dev(toks))
+    rsel, rw = ref.router_hash_select(logits, tid2eid, toks)
+    assert np.array_equal(sel.cpu().numpy(), rsel)
+    np.testing.assert_allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=1e-9)
+    # pinned routing: the layer computes with these picks and weights
+    s, wts = small_case(hidden=768, inter=256, E=8, k=3, seed=23)
+    from deepstrix_amd.executor import MoeLayer
+    T2 = 5
+    table = np.stack([rng.choice(s.n_expert, s.n_used, replace=False) for _ in range(16)]).astype(np.int32)
+    tk = rng.integers(0, 16, T2).astype(np.int32)
+    x, lg, _ = H.host_inputs(s, T2)
+    dsel = torch.zeros((T2, s.n_used), dtype=torch.int32, device="cuda")
+    dw = torch.zeros((T2, s.n_used), dtype=torch.float32, device="cuda")
+    dispatch.router_hash_select(dsel, dw, dev(lg), dev(table), dev(tk))
+    layer = MoeLayer(H.device_weights(s), T2)
+    out = layer.run(dev(x), None, selected_in=dsel, weights_in=dw)
+    hsel, hw = ref.router_hash_select(lg, table, tk)
+    want = ref.moe_forward(wts, x, hsel, hw)
+    assert H.max_rel(out.cpu().numpy(), want) < OUT_TOL
+
+
 def test_small_kernels_match_oracle():
     rng = np.random.default_rng(3)
     x = rng.standard_normal((5, 7168)).astype(np.float32)

@@ -98,6 +98,36 @@ def test_weight_sum_floor():
     np.testing.assert_allclose(w[0], p / eps * 1.5, rtol=1e-5)
 
 
+def test_hash_router_select_closed_form_floor_and_empty_slots():
+    # crates/v4flash-kernels/src/routing.rs:21-44: picks are the token's row of tid2eid,
+    # weights sqrt(softplus(logit)) / max(sum, 6.103515625e-5) * 1.5
+    rng = np.random.default_rng(11)
+    E, k, vocab, T = 256, 6, 50, 9
+    tid2eid = np.stack([rng.choice(E, k, replace=False) for _ in range(vocab)]).astype(np.int32)
+    toks = rng.integers(0, vocab, T).astype(np.int32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[4] = -30.0                                  # sum of p below the floor
+    sel, w = ref.router_hash_select(logits, tid2eid, toks)
+    assert np.array_equal(sel, tid2eid[toks])
+    p = np.take_along_axis(probs64(logits, SQRT_SOFTPLUS), sel.astype(np.int64), axis=1)
+    want = p / np.maximum(p.sum(axis=1, keepdims=True), 6.103515625e-5) * 1.5
+    np.testing.assert_allclose(w, want, rtol=2e-6)
+    np.testing.assert_allclose(np.delete(w, 4, axis=0).sum(axis=1), 1.5, rtol=1e-6)
+    assert w[4].sum() < 0.1
+    # with the learned router's own picks as the table, the weights are the learned router's
+    lsel, lw = ref.router_topk(logits, None, k, 1.5, 6.103515625e-5, SQRT_SOFTPLUS)
+    hsel, hw = ref.router_hash_select(logits, lsel, np.arange(T, dtype=np.int32))
+    assert np.array_equal(hsel, lsel) and np.array_equal(hw.view(np.uint32), lw.view(np.uint32))
+    # ids out of range leave empty slots
+    bad = tid2eid.copy()
+    bad[toks[0], 2] = E
+    bad[toks[0], 3] = -7
+    sel2, w2 = ref.router_hash_select(logits[:3], bad, np.concatenate([toks[:1], [vocab, -1]]).astype(np.int32))
+    assert sel2[0, 2] == -1 and sel2[0, 3] == -1 and w2[0, 2] == 0 and w2[0, 3] == 0
+    np.testing.assert_allclose(w2[0].sum(), 1.5, rtol=1e-6)
+    assert (sel2[1:] == -1).all() and (w2[1:] == 0).all()
+
+
 def test_softmax_matches_numpy():
     rng = np.random.default_rng(11)
     logits = rng.normal(0, 2, (16, 64)).astype(np.float32)
