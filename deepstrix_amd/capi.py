@@ -56,6 +56,7 @@ SIGNATURES = {
     "dsx_init": (_int, []),
     "dsx_router_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _f32, _u32, _u32, _u32, _u32]),
     "dsx_router_hash_select": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _f32, _f32, _u32]),
+    "dsx_moe_hetsplit_select": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "dsx_router_logits": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "dsx_router_logits_f16": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "dsx_q8k_quantize": (_int, [_vp, _vp, _vp, _u32]),

@@ -225,6 +225,20 @@ int dsx_router_hash_select(dsx_stream_t stream, int32_t *selected, float *weight
     return launched("router_hash_select");
 }
 
+int dsx_moe_hetsplit_select(dsx_stream_t stream, int32_t *selected_side, const int32_t *selected,
+                            const int32_t *remap, uint32_t mode, uint32_t cap, uint32_t n_used,
+                            uint32_t n_expert, uint32_t b) {
+    if (b == 0) return DSX_OK;
+    if (!selected_side || !selected || !remap)
+        return fail(DSX_ERR_INVALID_ARG, "moe_hetsplit_select: null pointer");
+    if (mode > 1) return fail(DSX_ERR_INVALID_ARG, "moe_hetsplit_select: mode=%u", mode);
+    if (n_used == 0 || n_expert == 0)
+        return fail(DSX_ERR_INVALID_ARG, "moe_hetsplit_select: n_used=%u n_expert=%u", n_used, n_expert);
+    hipLaunchKernelGGL(k_hetsplit_select, dim3((b + 255) / 256), dim3(256), 0, S(stream),
+                       selected_side, selected, remap, mode, cap, n_used, n_expert, b);
+    return launched("moe_hetsplit_select");
+}
+
 // ---- quantizers -----------------------------------------------------------------------
 int dsx_q8k_quantize(dsx_stream_t stream, uint8_t *out, const float *x, uint32_t n_blocks) {
     if (n_blocks == 0) return DSX_OK;

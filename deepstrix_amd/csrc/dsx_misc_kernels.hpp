@@ -248,6 +248,39 @@ __global__ __launch_bounds__(256) void k_router_hash_select(
         if (i < n_used) weights[(uint64_t)t * n_used + i] = w[i] / sum * scale;
 }
 
+// Het-split ownership (the rule of the reference's *_hetsplit kernels,
+// crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:231-284,
+// kernels/q2_k_accumulate_matvec_par.hip:731-766): remap[e] >= 0 is the dense slot of a
+// resident expert on the mode-1 side, -(slot + 1) the packed slot of a cold one; mode 1 takes
+// a token's first `cap` resident picks in slot order, mode 0 everything else.  out[b, s] is
+// the index this side's weight buffer is addressed with, or -1 (not this side's, or empty):
+// with it as `selected`, every entry point computes this side's share and zero-fills the rest.
+__global__ __launch_bounds__(256) void k_hetsplit_select(int32_t *__restrict__ out,
+                                                         const int32_t *__restrict__ selected,
+                                                         const int32_t *__restrict__ remap,
+                                                         uint32_t mode, uint32_t cap, uint32_t n_used,
+                                                         uint32_t n_expert, uint32_t n_tokens) {
+    const uint32_t b = blockIdx.x * 256u + threadIdx.x;
+    if (b >= n_tokens) return;
+    uint32_t rank = 0;
+    for (uint32_t s = 0; s < n_used; s++) {
+        const int e = selected[(uint64_t)b * n_used + s];
+        int r = -1;
+        if (e >= 0 && (uint32_t)e < n_expert) {
+            const int dense = remap[e];
+            const bool resident = dense >= 0;
+            const bool dgpu_takes = resident && rank < cap;
+            if (resident) rank++;
+            if (mode == 1u) {
+                if (dgpu_takes) r = dense;
+            } else if (!dgpu_takes) {
+                r = resident ? e : -dense - 1;
+            }
+        }
+        out[(uint64_t)b * n_used + s] = r;
+    }
+}
+
 // Front of the layer in one launch: workgroups [0, n_tokens) route one token each (skipped
 // when routing is pinned), the rest quantize the activations into staged rows (one wave per
 // 256-element block) and clear the arrival counters of the fused mid quantization.

@@ -55,6 +55,15 @@ def router_hash_select(selected, weights, logits, tid2eid, token_ids, scale=1.5,
                                        _p(token_ids), n_expert, n_used, vocab, scale, eps, b))
 
 
+def moe_hetsplit_select(selected_side, selected, remap, mode, cap):
+    """One side's picks under the reference's het-split rule
+    (crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:231-284); -1 = not this side's."""
+    capi.init()
+    b, n_used = selected.shape
+    check(lib().dsx_moe_hetsplit_select(_stream(), _p(selected_side), _p(selected), _p(remap), mode,
+                                        cap, n_used, remap.numel(), b))
+
+
 def router_logits(logits, router_w, x, n_expert, hidden, n_tokens):
     """crates/v4flash-kernels/kernels/laguna_ops.hip:57-60 (f32 W . x); f16 router weights as
     crates/v4flash-kernels/src/f16.rs:37-45 keeps them take the f16 entry point."""

@@ -167,6 +167,22 @@ int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, cons
                            uint32_t max_work_items, uint64_t dbpe, uint32_t xq_slot_stride,
                            uint32_t n_used, uint32_t chunk, uint32_t n_rows,
                            uint32_t n_blocks_in);
+/* The het-split variants (dispatch::moe_gate_up_batch_hetsplit, moe_down_batched_hetsplit,
+ * MoeGroupBuilder::launch_hetsplit, launch_reduce_partials_hetsplit;
+ * crates/v4flash-kernels/src/het/dispatch.rs:68-119,152-185,
+ * kernels/mxfp4_pair_matvec.hip:231-284, kernels/q2_k_accumulate_matvec_par.hip:731-766)
+ * share one ownership rule: remap[e] >= 0 is the dense slot of a resident expert on the
+ * mode-1 side, -(slot + 1) the packed slot of a cold one; mode 1 takes a token's first `cap`
+ * resident picks in slot order, mode 0 everything else.  This entry point applies the rule
+ * once: selected_side[b, n_used] = the index this side's weight buffer is addressed with, or
+ * -1 where the slot is the other side's (or empty).  Passed as `selected` to
+ * dsx_moe_gate_up_batch / dsx_moe_down_batched / dsx_moe_group_build /
+ * dsx_moe_reduce_partials / dsx_moe_layer_forward (selected_in), it makes each of them its
+ * het-split variant: slots not owned are zero-filled or skipped, so the two sides' results
+ * add up to the unsplit one. */
+int dsx_moe_hetsplit_select(dsx_stream_t stream, int32_t *selected_side, const int32_t *selected,
+                            const int32_t *remap, uint32_t mode, uint32_t cap, uint32_t n_used,
+                            uint32_t n_expert, uint32_t b);
 /* Q2KAccumulateMatvec::launch_reduce_partials (crates/v4flash-kernels/src/q2_k.rs:454-500;
  * kernels/q2_k_accumulate_matvec_par.hip:714-730): out[t,row] = sum over slots, in
  * slot order.  selected (nullable): slots with selected < 0 are skipped, so the

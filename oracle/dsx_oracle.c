@@ -622,6 +622,36 @@ void dsx_ref_router_hash_select(int32_t *selected, float *weights, const float *
     }
 }
 
+/* The het-split ownership rule shared by the reference's *_hetsplit kernels
+ * (K/kernels/mxfp4_pair_matvec.hip:231-284, K/kernels/q2_k_accumulate_matvec_par.hip:731-766):
+ * remap[e] >= 0 is the dense slot of a resident ("hot") expert on the dGPU side, -(slot + 1)
+ * the packed slot of a cold one.  The dGPU side (mode 1) takes the first `cap` resident picks
+ * of a token in slot order, the other side (mode 0) everything else.  out[b, s] = the expert
+ * index this side's weight buffer is addressed with, or -1 where the slot is not this side's
+ * (or is empty). */
+void dsx_ref_hetsplit_select(int32_t *out, const int32_t *selected, const int32_t *remap, int mode,
+                             int cap, int n_used, int n_expert, int n_tokens) {
+    for (int b = 0; b < n_tokens; b++) {
+        int rank = 0;
+        for (int s = 0; s < n_used; s++) {
+            const int e = selected[(size_t)b * n_used + s];
+            int r = -1;
+            if (e >= 0 && e < n_expert) {
+                const int dense = remap[e];
+                const int resident = dense >= 0;
+                const int dgpu_takes = resident && rank < cap;
+                if (resident) rank++;
+                if (mode == 1) {
+                    if (dgpu_takes) r = dense;
+                } else if (!dgpu_takes) {
+                    r = resident ? e : -dense - 1;
+                }
+            }
+            out[(size_t)b * n_used + s] = r;
+        }
+    }
+}
+
 /* K/kernels/laguna_ops.hip:57-60 */
 void dsx_ref_router_logits(float *logits, const float *w, const float *x, int n_expert,
                            int hidden, int n_tokens) {

@@ -99,6 +99,7 @@ def _declare(l):
     l.dsx_ref_router_scores.restype = i32
     l.dsx_ref_router_scores.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32]
     l.dsx_ref_router_logits.argtypes = [vp, vp, vp, i32, i32, i32]
+    l.dsx_ref_hetsplit_select.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32]
     l.dsx_ref_router_hash_select.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, i32]
     l.dsx_ref_group_build.restype = i32
     l.dsx_ref_group_build.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32]
@@ -287,6 +288,17 @@ def router_hash_select(logits, tid2eid, token_ids, scale=1.5, eps=6.103515625e-5
     lib().dsx_ref_router_hash_select(_p(sel), _p(w), _p(logits), _p(tid2eid), _p(token_ids), E,
                                      n_used, vocab, scale, eps, T)
     return sel, w
+
+
+def hetsplit_select(selected, remap, mode, cap):
+    """Per-slot expert index of one side of the reference's het-split, -1 where the slot is the
+    other side's (crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:231-284)."""
+    selected = _c(selected, np.int32)
+    remap = _c(remap, np.int32)
+    T, k = selected.shape
+    out = np.empty((T, k), np.int32)
+    lib().dsx_ref_hetsplit_select(_p(out), _p(selected), _p(remap), mode, cap, k, remap.size, T)
+    return out
 
 
 def router_scores(logits, bias, mode, n_group=1, topk_group=1):

@@ -264,6 +264,36 @@ def test_hash_router_select_matches_oracle_and_feeds_the_layer():
     assert H.max_rel(out.cpu().numpy(), want) < OUT_TOL
 
 
+@pytest.mark.parametrize("T", [1, 3, 40])
+def test_hetsplit_sides_add_up_to_the_unsplit_layer(T):
+    """The reference's het-split identity (crates/v4flash-kernels/tests/mxfp4_pair_oracle.rs:198-241):
+    out(side 0) + out(side 1) = out.  Both sides read the same weight buffer here (resident
+    experts keep their index as dense slot, cold ones are packed at their own index)."""
+    rng = np.random.default_rng(40 + T)
+    s = H.Shape(768, 256, 8, 3, shared=False, seed=25, clamp=10.0)
+    wts = H.host_weights(s)
+    from deepstrix_amd.executor import MoeLayer
+    layer = MoeLayer(H.device_weights(s), T)
+    x, lg, bias = H.host_inputs(s, T)
+    sel, w = H.oracle_route(s, lg, bias)
+    hot = rng.random(s.n_expert) < 0.5
+    remap = np.where(hot, np.arange(s.n_expert), -(np.arange(s.n_expert) + 1)).astype(np.int32)
+    dsel, dw, dx = dev(sel), dev(w), dev(x)
+    full = layer.run(dx, None, selected_in=dsel, weights_in=dw).cpu().numpy()
+    assert H.max_rel(full, ref.moe_forward(wts, x, sel, w)) < OUT_TOL
+    for cap in (1, 2):
+        parts = []
+        for mode in (0, 1):
+            side = torch.full((T, s.n_used), 77, dtype=torch.int32, device="cuda")
+            dispatch.moe_hetsplit_select(side, dsel, dev(remap), mode, cap)
+            want_side = ref.hetsplit_select(sel, remap, mode, cap)
+            assert np.array_equal(side.cpu().numpy(), want_side)
+            got = layer.run(dx, None, selected_in=side, weights_in=dw).cpu().numpy()
+            assert H.max_rel(got, ref.moe_forward(wts, x, want_side, w)) < OUT_TOL
+            parts.append(got)
+        assert H.max_rel(parts[0] + parts[1], full) < 1e-5
+
+
 def test_small_kernels_match_oracle():
     rng = np.random.default_rng(3)
     x = rng.standard_normal((5, 7168)).astype(np.float32)

@@ -128,6 +128,37 @@ def test_hash_router_select_closed_form_floor_and_empty_slots():
     assert (sel2[1:] == -1).all() and (w2[1:] == 0).all()
 
 
+def test_hetsplit_select_partitions_the_picks():
+    # crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:231-284: the two sides of the split
+    # own disjoint slots that together cover every pick; the mode-1 side owns the first `cap`
+    # resident picks of a token in slot order
+    rng = np.random.default_rng(31)
+    E, k, T = 40, 6, 200
+    remap = np.empty(E, np.int32)
+    hot = rng.random(E) < 0.5
+    remap[hot] = np.arange(hot.sum())                      # dense slots of the resident experts
+    remap[~hot] = -(np.arange((~hot).sum()) + 1)           # packed slots of the cold ones
+    sel = np.stack([rng.choice(E, k, replace=False) for _ in range(T)]).astype(np.int32)
+    sel[3, 2] = -1                                         # an empty slot belongs to nobody
+    for cap in (0, 1, 3, 6, 99):
+        a = ref.hetsplit_select(sel, remap, 0, cap)
+        b = ref.hetsplit_select(sel, remap, 1, cap)
+        owned_a, owned_b = a >= 0, b >= 0
+        assert not (owned_a & owned_b).any()
+        assert np.array_equal(owned_a | owned_b, sel >= 0)
+        for t in range(T):
+            resident_slots = [s_ for s_ in range(k) if sel[t, s_] >= 0 and hot[sel[t, s_]]]
+            want_b = resident_slots[:cap]
+            assert [s_ for s_ in range(k) if owned_b[t, s_]] == want_b
+            for s_ in range(k):
+                e = sel[t, s_]
+                if owned_b[t, s_]:
+                    assert b[t, s_] == remap[e]            # dense slot on the resident side
+                if owned_a[t, s_]:
+                    assert a[t, s_] == (e if hot[e] else -remap[e] - 1)
+    assert (ref.hetsplit_select(sel, remap, 1, 0) == -1).all()
+
+
 def test_softmax_matches_numpy():
     rng = np.random.default_rng(11)
     logits = rng.normal(0, 2, (16, 64)).astype(np.float32)
