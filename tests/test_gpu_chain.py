@@ -129,6 +129,34 @@ def test_small_chain_eager_and_graph():
             assert H.max_rel(eager.cpu().numpy(), want) < 3 * OUT_TOL   # three layers deep
 
 
+@pytest.mark.parametrize("T,fmt", [(16, "mxfp4"), (130, "mxfp4"), (16, "q8_0"), (130, "q8_0"), (130, "mixed")])
+def test_graph_replay_of_the_by_expert_and_gemm_paths(T, fmt):
+    """Every entry point is meant to be captured: the by-expert path (T = 16) and the grouped
+    GEMMs (T = 130), for MXFP4, Q8_0 and MXFP4 gate/up + Q8_0 down layers, replayed several times
+    with eager work of the same library in between; every replay must equal the eager step."""
+    from deepstrix_amd.capi import FMT_MXFP4, FMT_Q8_0
+    kw = dict(router_mode=1, route_scale=2.5, clamp=10.0, seed=121, shared=True)
+    if fmt == "q8_0":
+        kw.update(gate_fmt=FMT_Q8_0, down_fmt=FMT_Q8_0)
+    elif fmt == "mixed":   # like BASELINE config 5: MXFP4 gate/up, Q8_0 down, Q8_0 shared expert
+        kw.update(down_fmt=FMT_Q8_0, sh_gate_fmt=FMT_Q8_0, sh_down_fmt=FMT_Q8_0)
+    base = H.Shape(512, 256, 8, 2, **kw)
+    shapes = layer_shapes(base, 2)
+    chain = MoeChain([H.device_weights(s, block=True) for s in shapes], T)
+    rng = np.random.default_rng(T)
+    chain.capture(T)
+    for step in range(3):
+        h = rng.normal(0, 1, (T, base.hidden)).astype(np.float32)
+        eager = chain.step(torch.from_numpy(h).cuda()).clone()
+        torch.cuda.synchronize()
+        replayed = chain.replay(torch.from_numpy(h).cuda()).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(eager, replayed), f"graph replay {step} differs from the eager step"
+    want, min_gap = run_chain_oracle(shapes, h)
+    if min_gap > 1e-2:
+        assert H.max_rel(eager.cpu().numpy(), want) < 3 * OUT_TOL
+
+
 def test_config4_chain_of_v3_layers():
     """8 chained V3-shape MXFP4 layers, RMSNorm eps 1e-6 + residual, T = 2."""
     shapes = layer_shapes(H.CFG2, 8)
