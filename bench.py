@@ -222,7 +222,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the T=4096 prefill leg")
     ap.add_argument("--no-chain", action="store_true", help="skip the 8-layer chained decode leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the informative T=4/16/64 legs")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the informative legs: T=4/16/64 of config 2 and configs 5 and 1")
+    ap.add_argument("--no-small-t", action="store_true", help="skip only the T=4/16/64 legs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -314,7 +316,7 @@ def main():
              "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
              "layer_GBps_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9,
              "layer_frac_of_hbm_peak_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    for T in (() if args.no_extra else (4, 16, 64)):
+    for T in (() if (args.no_extra or args.no_small_t) else (4, 16, 64)):
         xs, ls, _ = H.host_inputs(H.Shape(**{**base.__dict__, "seed": base.seed + T}), T)
         xs, ls = torch.from_numpy(xs).cuda(), torch.from_numpy(ls).cuda()
         o = torch.empty((T, base.hidden), dtype=torch.float32, device="cuda")
