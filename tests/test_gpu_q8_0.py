@@ -180,6 +180,26 @@ def test_config1_router_logits_from_fp32_matvec():
     assert H.max_rel(out.cpu().numpy(), want) < OUT_TOL
 
 
+def test_config1_against_the_committed_fixture():
+    """tests/golden/cfg1_T4.npz: logits, picks, weights and layer output of config 1 at T = 4."""
+    import os
+    s, T = H.CFG1, 4
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cfg1_T4.npz"),
+                allow_pickle=False)
+    x, _, _ = H.host_inputs(s, T)
+    W = synth.normal_dev(s.seed, synth.T_ROUTER_W, s.n_expert * s.hidden, 0.02).reshape(s.n_expert, s.hidden)
+    dlog = torch.zeros((T, s.n_expert), dtype=torch.float32, device="cuda")
+    dispatch.router_logits(dlog, W, dev(x), s.n_expert, s.hidden, T)
+    np.testing.assert_allclose(dlog.cpu().numpy(), g["logits"], atol=2e-5)
+    layer = MoeLayer(H.device_weights(s), T)
+    out, sel, w = layer.run(dev(x), dlog, want_routing=True)
+    _, scores = ref.router_scores(g["logits"], None, s.router_mode)
+    assert H.routing_mismatch_explained(sel.cpu().numpy(), g["sel"], scores, s.n_used) == []
+    if np.array_equal(sel.cpu().numpy(), g["sel"]):
+        np.testing.assert_allclose(w.cpu().numpy(), g["w"], rtol=2e-5)
+        assert H.max_rel(out.cpu().numpy(), g["out"]) < OUT_TOL
+
+
 def test_mixed_precision_small_layer():
     s = H.Shape(512, 256, 8, 2, FMT_MXFP4, FMT_Q8_0, clamp=10.0, seed=35, route_scale=2.5)
     for T in (1, 7):

@@ -154,6 +154,23 @@ def test_expert_weight_is_applied_before_the_second_quantization():
 
 # ---- synthetic tensors ------------------------------------------------------------------
 
+def test_config1_fixture_is_what_the_oracle_computes():
+    """tests/golden/cfg1_T4.npz freezes the oracle's config-1 result (inputs from seeds)."""
+    import importlib.util
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_cfg1_fixture", os.path.join(here, "make_cfg1_fixture.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    now = mod.compute()
+    with np.load(os.path.join(here, "cfg1_T4.npz"), allow_pickle=False) as g:
+        assert np.array_equal(g["sel"], now["sel"])
+        # expf / logf of another libm may differ in the last bit; everything else is exact
+        np.testing.assert_allclose(now["logits"], g["logits"], rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(now["w"], g["w"], rtol=1e-6)
+        np.testing.assert_allclose(now["out"], g["out"], rtol=1e-5, atol=1e-7)
+
+
 def test_synth_normal_moments_and_determinism():
     a = synth.normal_host(1, synth.T_X, 1 << 16)
     b = synth.normal_host(1, synth.T_X, 1 << 16)
