@@ -124,6 +124,36 @@ def test_null_layer_handles_are_errors():
     l.dsx_moe_layer_destroy(None)  # a no-op, like free(NULL)
 
 
+def test_operators_refuse_bad_arguments_before_any_launch():
+    """Validation comes first in every entry point: these calls return an error code without a
+    device (pointers are fake; nothing is launched when the arguments are refused)."""
+    l = capi.lib()
+    p = 0x1000  # a non-null, 16-byte aligned stand-in
+    bad = [
+        l.dsx_router_topk(None, p, p, p, None, 0, 1, 1.0, 1e-20, 1, 0, 1, 1),          # n_expert = 0
+        l.dsx_router_topk(None, p, p, p, None, 64, 6, 1.0, 1e-20, 1, 3, 1, 1),         # mode 3
+        l.dsx_router_topk(None, p, p, p, None, 64, 6, 1.0, 1e-20, 1, 1, 7, 2),         # 64 % 7 != 0
+        l.dsx_router_hash_select(None, p, p, p, p, p, 64, 0, 10, 1.5, 6e-5, 1),        # n_used = 0
+        l.dsx_router_hash_select(None, p, p, p, None, p, 64, 6, 10, 1.5, 6e-5, 1),     # null table
+        l.dsx_moe_hetsplit_select(None, p, p, p, 2, 1, 6, 64, 1),                      # mode 2
+        l.dsx_moe_group_build(None, p, p, p, p, p, p, 4, 6, 64, 65),                   # chunk 65
+        l.dsx_moe_group_build(None, p, p, p, p, p, p, 70000, 6, 64, 4),                # b >= 65536
+        l.dsx_moe_gate_up_batch(None, capi.FMT_MXFP4, p, p, p, p, p, p, 8, 8, 6, 0.0, 24, 2),   # rows % 16
+        l.dsx_moe_gate_up_batch(None, 12, p, p, p, p, p, p, 8, 8, 6, 0.0, 32, 2),               # format id
+        l.dsx_moe_gate_up_chunked_rows(None, capi.FMT_MXFP4, p, p, p, p, p, p, p, p, p, p, 4, 8, 8, 6, 65,
+                                       0.0, 32, 2),                                              # chunk 65
+        l.dsx_moe_down_by_expert(None, capi.FMT_MXFP4, p, p, p, p, p, p, p, p, 4, 8, 292, 6, 0, 32, 1),  # chunk 0
+        l.dsx_q8_0_weights_from_hf(None, p, p, None, capi.SRC_F8E4M3, 64, 64, 0, 0, 1),   # fp8 without scales
+        l.dsx_q8_0_weights_from_hf(None, p, p, p, capi.SRC_F8E4M3, 64, 64, 3, 2, 1),      # grid does not tile
+        l.dsx_q8_0_weights_from_hf(None, p, p, None, capi.SRC_F32, 64, 48, 0, 0, 1),      # cols % 32
+        l.dsx_q8_0_repack_rows(None, p, p, 4, 2),                                          # in place
+        l.dsx_mxfp4_repack_hf_to_v2(None, p, p, p, 4, 7),                                  # nb % 8
+        l.dsx_rms_norm(None, p, p, None, 64, 1e-6, 1) if hasattr(l, "dsx_rms_norm") else -1,
+    ]
+    assert all(rc < 0 for rc in bad), bad
+    assert l.dsx_last_error()
+
+
 def test_missing_library_is_an_import_error_not_a_fallback(monkeypatch):
     monkeypatch.setattr(capi, "_lib", None)
     monkeypatch.setattr(capi, "LIB_PATH", os.path.join(ROOT, "deepstrix_amd", "lib", "absent.so"))
