@@ -31,6 +31,112 @@ __device__ __forceinline__ float softplus_stable(float x) {
 
 constexpr int kRouterThreads = 256;
 
+// ---- one-wave router ----------------------------------------------------------------------
+// With 64 C experts (C = 1, 2, 4, 8) one wave routes a token without LDS or barriers: lane l
+// owns experts C l .. C l + C - 1, the arg-max of each of the k passes is a 64-bit key
+// (score, ~index) reduced with DPP moves (wave_max_u64_dpp), the winner is cleared and the
+// next pass follows.
+// Same picks and weights as the workgroup-wide version below (ties -> lowest index, weights
+// summed in pick order).
+// Whether the one-wave router takes this shape (softmax keeps the workgroup-wide version).
+__device__ __forceinline__ bool route_wave_ok(uint32_t n_expert, uint32_t mode, uint32_t n_group,
+                                              uint32_t topk_group) {
+    if (mode == 2u || n_expert % 64u != 0u) return false;
+    const uint32_t c = n_expert / 64u;
+    if (c != 1u && c != 2u && c != 4u && c != 8u) return false;
+    if (n_group > 1u && topk_group < n_group) {
+        if (n_expert % n_group != 0u) return false;
+        const uint32_t gs = n_expert / n_group;
+        if (gs % c != 0u) return false;
+        const uint32_t lg = gs / c;  // lanes per group
+        if ((lg & (lg - 1u)) != 0u) return false;
+    }
+    return true;
+}
+
+template <int C>
+__device__ __forceinline__ void route_token_wave(int32_t *__restrict__ selected,
+                                                 float *__restrict__ weights,
+                                                 const float *__restrict__ lg,
+                                                 const float *__restrict__ bias, uint32_t n_expert,
+                                                 uint32_t n_used, float scale, float eps, uint32_t mode,
+                                                 uint32_t n_group, uint32_t topk_group) {
+    const uint32_t lane = threadIdx.x & 63u;
+    float p[C], s[C];
+#pragma unroll
+    for (int i = 0; i < C; i++) p[i] = lg[lane * C + i];
+#pragma unroll
+    for (int i = 0; i < C; i++) {
+        p[i] = (mode == 0u) ? sqrtf(softplus_stable(p[i])) : 1.0f / (1.0f + expf(-p[i]));
+        s[i] = (bias != nullptr) ? p[i] + bias[lane * C + i] : p[i];
+    }
+    if (n_group > 1u && topk_group < n_group) {
+        // group score = sum of the two largest biased scores of the group (lanes_per_group
+        // consecutive lanes), groups ranked with ties to the lower index
+        const uint32_t gs = n_expert / n_group, lanes_per_group = gs / C;
+        float a = -INFINITY, b = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            const float v = s[i];
+            b = fmaxf(fminf(a, v), b);
+            a = fmaxf(a, v);
+        }
+        for (uint32_t off = 1; off < lanes_per_group; off <<= 1) {
+            const float oa = __shfl_xor(a, (int)off, 64), ob = __shfl_xor(b, (int)off, 64);
+            const float hi = fmaxf(a, oa), lo = fminf(a, oa);
+            b = fmaxf(lo, fmaxf(b, ob));
+            a = hi;
+        }
+        const float mine = (gs >= 2u) ? a + b : a;
+        const uint32_t my_group = lane / lanes_per_group;
+        uint32_t rank = 0;
+        for (uint32_t g = 0; g < n_group; g++) {
+            const float o = __shfl(mine, (int)(g * lanes_per_group), 64);
+            rank += (o > mine || (o == mine && g < my_group)) ? 1u : 0u;
+        }
+        if (rank >= topk_group) {
+#pragma unroll
+            for (int i = 0; i < C; i++) s[i] = -INFINITY;
+        }
+    }
+    uint64_t key[C];
+#pragma unroll
+    for (int i = 0; i < C; i++)
+        key[i] = (s[i] > -INFINITY) ? (((uint64_t)f32_key(s[i]) << 32) | (uint64_t)(0xFFFFFFFFu - (lane * C + i)))
+                                    : 0ull;  // a masked expert is never picked
+    int my_sel = -1;
+    float my_p = 0.0f;
+    for (uint32_t j = 0; j < n_used; j++) {
+        uint64_t best = key[0];
+#pragma unroll
+        for (int i = 1; i < C; i++) best = key[i] > best ? key[i] : best;
+        const uint64_t top = wave_max_u64_dpp(best);  // uniform
+        if (top == 0ull) break;                       // fewer eligible experts than picks
+        const uint32_t e = 0xFFFFFFFFu - (uint32_t)top;
+        float pw = 0.0f;
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            if (key[i] == top) {  // only the winner's lane, only its winning value
+                pw = p[i];
+                key[i] = 0ull;
+            }
+        }
+        pw = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(pw), (int)(e / C)));
+        if (lane == j) {
+            my_sel = (int)e;
+            my_p = pw;
+        }
+    }
+    float sum = 0.0f;
+    for (uint32_t j = 0; j < n_used; j++)  // pick order, as the reference
+        sum += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(my_p), (int)j));
+    if (sum < eps) sum = eps;
+    if (lane < n_used) {
+        selected[lane] = my_sel;
+        weights[lane] = my_p / sum * scale;
+    }
+}
+
 // One workgroup routes one token.  Thread t owns experts t and t + 256.  The top-k is read
 // off each expert's rank (how many experts beat it: larger score, or equal score and lower
 // index), which every thread counts on its own from 64-bit keys (score, ~index) in LDS.
@@ -49,6 +155,17 @@ __device__ __forceinline__ void route_token(int32_t *__restrict__ selected,
     __shared__ int s_esel[DSX_MAX_USED_K];
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    if (route_wave_ok(n_expert, mode, n_group, topk_group)) {  // uniform over the workgroup
+        if (wave == 0) {
+            switch (n_expert / 64u) {
+                case 1: route_token_wave<1>(selected, weights, lg, bias, n_expert, n_used, scale, eps, mode, n_group, topk_group); break;
+                case 2: route_token_wave<2>(selected, weights, lg, bias, n_expert, n_used, scale, eps, mode, n_group, topk_group); break;
+                case 4: route_token_wave<4>(selected, weights, lg, bias, n_expert, n_used, scale, eps, mode, n_group, topk_group); break;
+                default: route_token_wave<8>(selected, weights, lg, bias, n_expert, n_used, scale, eps, mode, n_group, topk_group); break;
+            }
+        }
+        return;
+    }
     const uint32_t nj = (n_expert + kRouterThreads - 1) / kRouterThreads;  // 1 or 2
     float p[2], s[2];
     float mx = -INFINITY;

@@ -9,6 +9,35 @@
 
 namespace dsx {
 
+// 64-lane maximum of a 64-bit key with data-parallel-primitive moves: four steps inside each
+// row of 16 lanes, two broadcasts across the rows, the result read from lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp_mov_u64(uint64_t v) {
+    const int lo = __builtin_amdgcn_update_dpp((int)(uint32_t)v, (int)(uint32_t)v, CTRL, ROW_MASK, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp((int)(uint32_t)(v >> 32), (int)(uint32_t)(v >> 32), CTRL,
+                                               ROW_MASK, 0xf, false);
+    return ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo;
+}
+// Maximum over the 64 lanes, returned to every lane (all lanes must be active).
+__device__ __forceinline__ uint64_t wave_max_u64_dpp(uint64_t v) {
+    uint64_t o;
+    o = dpp_mov_u64<0xb1, 0xf>(v);   // quad_perm:[1,0,3,2]
+    v = o > v ? o : v;
+    o = dpp_mov_u64<0x4e, 0xf>(v);   // quad_perm:[2,3,0,1]
+    v = o > v ? o : v;
+    o = dpp_mov_u64<0x124, 0xf>(v);  // row_ror:4
+    v = o > v ? o : v;
+    o = dpp_mov_u64<0x128, 0xf>(v);  // row_ror:8: every lane holds its row's maximum
+    v = o > v ? o : v;
+    o = dpp_mov_u64<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v = o > v ? o : v;
+    o = dpp_mov_u64<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3: lane 63 holds the maximum
+    v = o > v ? o : v;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
+    return ((uint64_t)hi << 32) | lo;
+}
+
 // 64-lane butterfly reductions.  Every lane ends with the full result.
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
 #pragma unroll
@@ -52,14 +81,14 @@ __device__ __forceinline__ Q8kQuant q8k_quantize_lane(float4 v, uint32_t lane) {
         const uint64_t key = ((uint64_t)(__float_as_uint(xs[i]) & 0x7FFFFFFFu) << 32) | (255u - idx);
         best = key > best ? key : best;
     }
-    best = wave_max_u64(best);
+    best = wave_max_u64_dpp(best);  // uniform; every lane of the wave is active here
     const uint32_t amax_bits = (uint32_t)(best >> 32);
     const uint32_t idx = 255u - (uint32_t)(best & 0xFFu);
     float cand = xs[0];
     if ((idx & 3u) == 1u) cand = xs[1];
     if ((idx & 3u) == 2u) cand = xs[2];
     if ((idx & 3u) == 3u) cand = xs[3];
-    const float mxv = __shfl(cand, (int)(idx >> 2), 64);
+    const float mxv = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cand), (int)(idx >> 2)));
     Q8kQuant r;
     if (amax_bits == 0u) {
         r.d = 0.0f;
