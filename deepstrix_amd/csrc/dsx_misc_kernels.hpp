@@ -81,17 +81,26 @@ __device__ __forceinline__ void route_token_wave(int32_t *__restrict__ selected,
             b = fmaxf(fminf(a, v), b);
             a = fmaxf(a, v);
         }
-        for (uint32_t off = 1; off < lanes_per_group; off <<= 1) {
-            const float oa = __shfl_xor(a, (int)off, 64), ob = __shfl_xor(b, (int)off, 64);
+        // lanes 2^j apart exchange their pairs; up to 16 lanes per group with DPP moves (after
+        // the steps before it every lane of a half holds the half's pair, so a mirror of 8 or
+        // 16 lanes reaches the other half like an exchange would)
+        auto merge = [&](float oa, float ob) {
             const float hi = fmaxf(a, oa), lo = fminf(a, oa);
             b = fmaxf(lo, fmaxf(b, ob));
             a = hi;
-        }
+        };
+        if (lanes_per_group > 1u) merge(dpp_mov_f32<0xb1>(a), dpp_mov_f32<0xb1>(b));    // quad_perm:[1,0,3,2]
+        if (lanes_per_group > 2u) merge(dpp_mov_f32<0x4e>(a), dpp_mov_f32<0x4e>(b));    // quad_perm:[2,3,0,1]
+        if (lanes_per_group > 4u) merge(dpp_mov_f32<0x141>(a), dpp_mov_f32<0x141>(b));  // row_half_mirror
+        if (lanes_per_group > 8u) merge(dpp_mov_f32<0x140>(a), dpp_mov_f32<0x140>(b));  // row_mirror
+        for (uint32_t off = 16; off < lanes_per_group; off <<= 1)
+            merge(__shfl_xor(a, (int)off, 64), __shfl_xor(b, (int)off, 64));
         const float mine = (gs >= 2u) ? a + b : a;
         const uint32_t my_group = lane / lanes_per_group;
         uint32_t rank = 0;
-        for (uint32_t g = 0; g < n_group; g++) {
-            const float o = __shfl(mine, (int)(g * lanes_per_group), 64);
+        for (uint32_t g = 0; g < n_group; g++) {  // g * lanes_per_group is uniform
+            const float o = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+                (int)__float_as_uint(mine), (int)(g * lanes_per_group)));
             rank += (o > mine || (o == mine && g < my_group)) ? 1u : 0u;
         }
         if (rank >= topk_group) {

@@ -18,6 +18,11 @@ __device__ __forceinline__ uint64_t dpp_mov_u64(uint64_t v) {
                                                ROW_MASK, 0xf, false);
     return ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo;
 }
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov_f32(float v) {
+    const int b = (int)__float_as_uint(v);
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(b, b, CTRL, 0xf, 0xf, false));
+}
 // Maximum over the 64 lanes, returned to every lane (all lanes must be active).
 __device__ __forceinline__ uint64_t wave_max_u64_dpp(uint64_t v) {
     uint64_t o;
