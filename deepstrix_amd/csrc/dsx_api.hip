@@ -69,8 +69,10 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gate_up<2, true, true, false>);
         allow_lds(k_mxfp4_gate_up<4, true, true, false>);
         allow_lds(k_mxfp4_gate_up<8, true, true, false>);
-        allow_lds(k_mxfp4_gemm<true>);
-        allow_lds(k_mxfp4_gemm<false>);
+        allow_lds(k_mxfp4_gemm<true, kGemmMT>);
+        allow_lds(k_mxfp4_gemm<false, kGemmMT>);
+        allow_lds(k_mxfp4_gemm<true, kGemmMTNarrow>);
+        allow_lds(k_mxfp4_gemm<false, kGemmMTNarrow>);
         allow_lds(k_mxfp4_down_decode<false>);
         allow_lds(k_mxfp4_down_decode<true>);
         allow_lds(k_mxfp4_down_by_expert<1, false>);
@@ -142,8 +144,9 @@ int group_build_big(hipStream_t st, int32_t *group_count, int32_t *group_offset,
     return launched("group_scatter");
 }
 
-// Grouped GEMM launch; max_wi bounds the number of work items.
-template <bool PAIR>
+// Grouped GEMM launch; max_wi bounds the number of work items, MT is the chunk they were built
+// with (kGemmMT or kGemmMTNarrow).
+template <bool PAIR, int MT = kGemmMT>
 int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
     if (max_wi == 0) return DSX_OK;
     const uint32_t per_xcd = (max_wi + 7u) / 8u;
@@ -154,8 +157,8 @@ int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
     if ((uint64_t)p.n_rows * p.n_sb * kSuperBytes > 0xFFFFFFFFull ||
         act_rows * p.act_row_bytes > 0xFFFFFFFFull)
         return fail(DSX_ERR_INVALID_ARG, "gemm: a weight matrix or the activation rows exceed 4 GiB");
-    hipLaunchKernelGGL((k_mxfp4_gemm<PAIR>), dim3((uint32_t)grid), dim3(kGemmWaves * 64), kGemmLdsBytes,
-                       st, p);
+    hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
+                       gemm_lds_bytes(MT), st, p);
     return launched(PAIR ? "gate_up gemm" : "down gemm");
 }
 

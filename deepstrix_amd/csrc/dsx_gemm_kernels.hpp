@@ -33,13 +33,15 @@ namespace dsx {
 
 constexpr int kGemmWaves = 8;
 constexpr int kGemmRF = 2;                  // 16-row fragments per wave and row set
-constexpr int kGemmMT = 128;                // token columns per workgroup
-constexpr int kGemmCG = kGemmMT / 16;       // column groups
-constexpr int kGemmHalfBytes = kGemmMT * 256;  // half a super-block of all columns in LDS
+constexpr int kGemmMT = 128;                // token columns per workgroup (the wide tile)
+constexpr int kGemmMTNarrow = 16;           // ... of the narrow tile: groups of a few members
 constexpr int kGemmAWaveBytes = 2 * kGemmRF * 2048 + 2 * 256;  // a wave's weights of one super-block
-constexpr int kGemmYdOff = 2 * kGemmHalfBytes;
-constexpr int kGemmAOff = kGemmYdOff + 2 * kGemmMT * (int)sizeof(float);
-constexpr size_t kGemmLdsBytes = kGemmAOff + kGemmWaves * kGemmAWaveBytes;
+// LDS of a workgroup with MT columns: two half super-blocks of the columns | two rows of 128
+// block scales (the loads that fill them are 64 lanes wide) | the waves' weight regions
+constexpr int gemm_half_bytes(int mt) { return mt * 256; }
+constexpr int gemm_yd_off(int mt) { return 2 * gemm_half_bytes(mt); }
+constexpr int gemm_a_off(int mt) { return gemm_yd_off(mt) + 2 * 128 * (int)sizeof(float); }
+constexpr size_t gemm_lds_bytes(int mt) { return (size_t)gemm_a_off(mt) + kGemmWaves * kGemmAWaveBytes; }
 
 struct GemmParams {
     const uint8_t *w0, *w1;        // [n_expert] experts (gate, up), or down in w0 (w1 unused)
@@ -66,14 +68,22 @@ __device__ __forceinline__ uint32_t gemm_dest_row(uint32_t m, uint32_t n_tokens,
     return slot >= n_used ? n_tokens * n_used + t : t * n_used + slot;
 }
 
-template <bool PAIR>
-__global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams p) {
+// MT = 128: one workgroup per CU (256 registers per lane).  MT = 16: an eighth of the
+// accumulators and of the column LDS, so that two workgroups share a CU (the second template
+// argument of the launch bounds asks for four waves per SIMD) -- with few members per group the
+// kernel only streams weights, and two workgroups keep twice the weight loads in flight.
+template <bool PAIR, int MT>
+__global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp4_gemm(const GemmParams p) {
+    constexpr int kGemmCG = MT / 16;                    // column groups
+    constexpr int kGemmHalfBytes = gemm_half_bytes(MT);  // half a super-block of all columns in LDS
+    constexpr int kGemmYdOff = gemm_yd_off(MT);
+    constexpr int kGemmAOff = gemm_a_off(MT);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ uint32_t s_dest[kGemmMT];
-    __shared__ uint32_t s_src[kGemmMT];
-    __shared__ float s_ew[kGemmMT];
-    __shared__ uint64_t s_key[kGemmWaves][kGemmMT];
-    __shared__ float s_iscale[kGemmMT];
+    __shared__ uint32_t s_dest[MT];
+    __shared__ uint32_t s_src[MT];
+    __shared__ float s_ew[MT];
+    __shared__ uint64_t s_key[kGemmWaves][MT];
+    __shared__ float s_iscale[MT];
 
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + kGemmYdOff);
@@ -96,11 +106,11 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
 
     const uint32_t wi = (uint32_t)p.work_items[item];
     const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
-    const uint32_t cnt = min((uint32_t)kGemmMT, (uint32_t)p.group_count[e] - start);
+    const uint32_t cnt = min((uint32_t)MT, (uint32_t)p.group_count[e] - start);
     const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
     const bool extra = e >= p.n_expert;
     const float clamp = extra ? p.sh_clamp : p.clamp;
-    if (tid < (uint32_t)kGemmMT) {
+    if (tid < (uint32_t)MT) {
         // columns past the end of the group repeat its last member; they are never stored
         const uint32_t m = (uint32_t)p.members[mbase + min(tid, cnt - 1u)];
         const uint32_t dest = gemm_dest_row(m, p.n_tokens, p.n_used);
@@ -192,8 +202,8 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     uint32_t b_fetch[2];  // column 16 w + 8 ii + l8, chunk c8 of each 128-byte run
 #pragma unroll
     for (int ii = 0; ii < 2; ii++)
-        b_fetch[ii] = s_src[wave * 16u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
-    const uint32_t yd_fetch = s_src[tid & (kGemmMT - 1)] * p.act_row_bytes + p.n_sb * 512u;
+        b_fetch[ii] = s_src[(wave * 16u + ii * 8u + l8) & (uint32_t)(MT - 1)] * p.act_row_bytes + c8 * 16u;
+    const uint32_t yd_fetch = s_src[tid & (uint32_t)(MT - 1)] * p.act_row_bytes + p.n_sb * 512u;
     const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 256u);
     // a wave whose 16 columns lie past the end of a short group fetches nothing (nobody reads
     // them: the column loop stops at the last group that holds a real column)
@@ -208,7 +218,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
                           b_fetch[ii] + sb * 512u + h * 256u + (uint32_t)q * 128u);
     };
     auto issue_yd = [&](uint32_t sb) {  // waves 0 and 1: 64 columns each
-        if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * (kGemmMT * 4u), p.act, yd_fetch + sb * 4u);
+        if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * 512u, p.act, yd_fetch + sb * 4u);
     };
 
     issue_b(0, 0);
@@ -233,7 +243,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     auto compute_half = [&](auto hc, const uint32_t sb) {
         constexpr int h = decltype(hc)::value;
         const uint8_t *half = tiles + h * kGemmHalfBytes;
-        const float *yds = s_yd + (sb & 1u) * kGemmMT;
+        const float *yds = s_yd + (sb & 1u) * 128u;
         auto load_piece = [&](int j, int q) -> v8i {
             const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 2u + (uint32_t)q) * 1024u + sw;
             return b_operand(half, cb, cb ^ 64u);
@@ -385,7 +395,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void k_mxfp4_gemm(const GemmParams
     if (p.midq == nullptr) return;  // f32 mid only (a down matrix of another format follows)
     __syncthreads();
     const uint32_t n_blk_out = p.n_rows / 256u;
-    if (tid < (uint32_t)kGemmMT) {
+    if (tid < (uint32_t)MT) {
         uint64_t k = s_key[0][tid];
 #pragma unroll
         for (int w = 1; w < kGemmWaves; w++) k = s_key[w][tid] > k ? s_key[w][tid] : k;

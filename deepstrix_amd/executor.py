@@ -98,10 +98,11 @@ class MoeLayer:
         """hipEvent_t handles (ints) recorded around the gate/up launch and after down."""
         check(lib().dsx_moe_layer_set_profile_events(self._h, gate_up_begin, gate_up_end, down_end))
 
-    def set_tuning(self, by_expert_chunk: int = 0, gemm_min_tokens: int = 0, decode_max_tokens: int = 0):
+    def set_tuning(self, by_expert_chunk: int = 0, gemm_min_tokens: int = 0, decode_max_tokens: int = 0,
+                   gemm_narrow_members: int = 0):
         """0 keeps the current value (include/dsx_moe.h: dsx_moe_layer_set_tuning)."""
         check(lib().dsx_moe_layer_set_tuning(self._h, by_expert_chunk, gemm_min_tokens,
-                                             decode_max_tokens))
+                                             decode_max_tokens, gemm_narrow_members))
 
     def block(self, h: torch.Tensor) -> torch.Tensor:
         """In place: h += layer(RMSNorm(h)), router logits = router_w . RMSNorm(h)

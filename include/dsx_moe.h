@@ -275,9 +275,12 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
  * path (128 token columns per work item, shared expert as an extra group; a Q8_0 down matrix
  * takes the int8 grouped GEMM).
  * decode_max_tokens: up to this many tokens, an all-MXFP4 layer runs the one-token decode
- * kernels once per token inside the same launches (no grouping by expert). */
+ * kernels once per token inside the same launches (no grouping by expert).
+ * gemm_narrow_members: while the picks per expert average less than this, the all-MXFP4
+ * grouped GEMMs use 16 token columns per work item and two workgroups per CU (they only
+ * stream weights then); 1 turns the narrow tile off. */
 int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
-                             uint32_t decode_max_tokens);
+                             uint32_t decode_max_tokens, uint32_t gemm_narrow_members);
 /* Bytes of caller-provided device scratch for up to max_tokens tokens. */
 size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
 /* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],

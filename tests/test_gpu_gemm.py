@@ -50,6 +50,27 @@ def test_small_layer_gemm_path(T):
     assert H.max_rel(got, base) < BASE_TOL
 
 
+@pytest.mark.parametrize("T", [40, 130])
+@pytest.mark.parametrize("narrow", [1, 1 << 20])
+def test_both_gemm_tiles_on_the_same_inputs(T, narrow):
+    """The 128-column tile (gemm_narrow_members = 1: never narrow) and the 16-column tile
+    (always narrow: groups of more than 16 members become several work items) agree with the
+    oracle and with the by-expert path."""
+    s = H.Shape(1024, 512, 16, 4, router_mode=1, route_scale=2.5, clamp=10.0, seed=95)
+    x, logits, bias = H.host_inputs(s, T)
+    layer = MoeLayer(H.device_weights(s), T)
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    layer.set_tuning(gemm_min_tokens=1 << 30)
+    base, sel, w = layer.run(dx, dl, want_routing=True)
+    base = base.clone()
+    layer.set_tuning(gemm_min_tokens=1, gemm_narrow_members=narrow)
+    got = layer.run(dx, None, selected_in=sel, weights_in=w).cpu().numpy()
+    sel_h, w_h = sel.cpu().numpy(), w.cpu().numpy()
+    want = ref.moe_forward(H.host_weights(s, experts=np.unique(sel_h)), x, sel_h, w_h)
+    assert H.max_rel(got, want) < OUT_TOL
+    assert H.max_rel(got, base.cpu().numpy()) < BASE_TOL
+
+
 def test_gemm_path_without_shared_expert():
     s = H.Shape(512, 256, 8, 2, shared=False, router_mode=0, route_scale=1.5,
                 route_eps=6.103515625e-5, seed=92)
