@@ -86,6 +86,7 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_down_by_expert<8, true>);
         allow_lds(k_mxfp4_down_by_expert<16, true>);
         q8_0_raise_lds_limits();
+        q8_0_gemm_raise_lds_limits();
     }
 }
 

@@ -613,6 +613,12 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
     }
 }
 
+// Raised once per device by the library's set-up, with the device current.
+inline void q8_0_gemm_raise_lds_limits() {
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gemm<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gemm<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+}
+
 template <bool PAIR>
 inline int q8_0_gemm(hipStream_t st, const Q8GemmParams &p, uint32_t max_wi) {
     if (max_wi == 0) return DSX_OK;
@@ -626,9 +632,6 @@ inline int q8_0_gemm(hipStream_t st, const Q8GemmParams &p, uint32_t max_wi) {
     const uint32_t per_xcd = (max_wi + 7u) / 8u;
     const uint64_t grid = (uint64_t)8u * per_xcd * p.n_row_tiles;
     if (grid > 0x7FFFFFFFull) return q8_0_fail(DSX_ERR_INVALID_ARG, "q8_0 gemm", "grid too large");
-    static const hipError_t attr = hipFuncSetAttribute((const void *)k_q8_0_gemm<PAIR>,
-                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
-    (void)attr;
     hipLaunchKernelGGL(k_q8_0_gemm<PAIR>, dim3((uint32_t)grid), dim3(kQgWaves * 64), lds, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? DSX_OK : q8_0_fail((int)e, "q8_0 gemm", hipGetErrorString(e));
