@@ -666,31 +666,62 @@ __global__ __launch_bounds__(256) void k_group_scatter(int32_t *__restrict__ mem
         for (uint32_t t = tid; t < b; t += 256u) members[base + t] = (int)((t << 16) | n_used);
         return;
     }
-    // each wave owns a quarter of the picks (rounded to 64): count, then place
+    // each wave owns a quarter of the picks (rounded to 256): count, then place; a lane looks at
+    // four consecutive picks per step (one 16-byte load when `selected` is aligned for it)
     const uint32_t total = b * n_used;
-    const uint32_t quarter = ((total + 255u) / 256u) * 64u;
-    const uint32_t i_begin = wave * quarter, i_end = min(total, i_begin + quarter);
+    const bool vec = ((uintptr_t)selected & 15u) == 0u;
+    const uint32_t quarter = ((total + 1023u) / 1024u) * 256u;
+    const uint32_t i_begin = min(total, wave * quarter), i_end = min(total, i_begin + quarter);
+    auto load4 = [&](uint32_t i0) -> int4 {  // picks i0 + 4 lane + j, -1 past the end
+        const uint32_t i = i0 + lane * 4u;
+        int4 q = {-1, -1, -1, -1};
+        if (vec && i + 4u <= i_end) {
+            q = *(const int4 *)(selected + i);
+        } else {
+            if (i < i_end) q.x = selected[i];
+            if (i + 1u < i_end) q.y = selected[i + 1u];
+            if (i + 2u < i_end) q.z = selected[i + 2u];
+            if (i + 3u < i_end) q.w = selected[i + 3u];
+        }
+        return q;
+    };
+    // the next step's picks are requested before this step's are counted
     uint32_t mine = 0;
-    for (uint32_t i0 = i_begin; i0 < i_end; i0 += 64u) {
-        const uint32_t i = i0 + lane;
-        const bool hit = (i < i_end) && (selected[i] == (int)e);
-        mine += (uint32_t)__popcll(__ballot(hit));
+    int4 cur = load4(i_begin);
+    for (uint32_t i0 = i_begin; i0 < i_end; i0 += 256u) {
+        const int4 nxt = load4(i0 + 256u);
+        mine += (uint32_t)__popcll(__ballot(cur.x == (int)e)) + (uint32_t)__popcll(__ballot(cur.y == (int)e)) +
+                (uint32_t)__popcll(__ballot(cur.z == (int)e)) + (uint32_t)__popcll(__ballot(cur.w == (int)e));
+        cur = nxt;
     }
     if (lane == 0) s_cnt[wave] = mine;
     __syncthreads();
     uint32_t pos = base;
     for (uint32_t w = 0; w < wave; w++) pos += s_cnt[w];
     if (mine == 0u) return;
-    for (uint32_t i0 = i_begin; i0 < i_end; i0 += 64u) {
-        const uint32_t i = i0 + lane;
-        const bool hit = (i < i_end) && (selected[i] == (int)e);
-        const uint64_t mask = __ballot(hit);
-        if (hit) {
-            const uint32_t before = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-            const uint32_t t = i / n_used, slot = i - t * n_used;
-            members[pos + before] = (int)((t << 16) | slot);
+    const uint64_t lower = (1ull << lane) - 1ull;
+    cur = load4(i_begin);
+    for (uint32_t i0 = i_begin; i0 < i_end; i0 += 256u) {
+        const int4 nxt = load4(i0 + 256u);
+        const bool h[4] = {cur.x == (int)e, cur.y == (int)e, cur.z == (int)e, cur.w == (int)e};
+        uint32_t before = 0, all = 0;
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const uint64_t mask = __ballot(h[jj]);
+            before += (uint32_t)__popcll(mask & lower);
+            all += (uint32_t)__popcll(mask);
         }
-        pos += (uint32_t)__popcll(mask);
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            if (h[jj]) {  // ascending pick index: lower lanes first, then the lane's own earlier picks
+                const uint32_t i = i0 + lane * 4u + jj;
+                const uint32_t t = i / n_used, slot = i - t * n_used;
+                members[pos + before] = (int)((t << 16) | slot);
+                before++;
+            }
+        }
+        pos += all;
+        cur = nxt;
     }
 }
 

@@ -181,6 +181,11 @@ def test_group_build_matches_oracle(T, E, k, chunk):
     assert np.array_equal(d_gc.cpu().numpy(), gc)
     assert np.array_equal(d_off.cpu().numpy(), off)
     assert np.array_equal(d_mem.cpu().numpy()[: mem.size], mem)
+    # the same picks from a buffer that is only 4-byte aligned (no 16-byte loads then)
+    shifted = dev(np.concatenate([np.zeros(1, np.int32), sel.ravel()]))[1:]
+    d_mem2 = torch.full((T * k,), -1, dtype=torch.int32, device="cuda")
+    dispatch.moe_group_build(d_gc, d_off, d_mem2, d_wi, d_n, shifted, T, k, E, chunk)
+    assert np.array_equal(d_mem2.cpu().numpy()[: mem.size], mem)
     n = int(d_n.item())
     assert n == wi.size and n <= dispatch.wi_upper_bound(T * k, E, chunk)
     assert np.array_equal(d_wi.cpu().numpy()[:n], wi)
