@@ -440,11 +440,19 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
     // one wave per 256-element block, grid-stride (many tokens: a few thousand workgroups
     // instead of one per four blocks)
     const uint32_t n_q = gridDim.x - n_route;
-    for (uint32_t blk = qb * 4u + (tid >> 6); blk < p.n_tokens * p.n_sb; blk += n_q * 4u) {
+    // (x rows are contiguous: block blk starts at element 256 blk); the next block's elements are
+    // requested before this one is quantized
+    const uint32_t n_blk = p.n_tokens * p.n_sb, step = n_q * 4u;
+    uint32_t blk = qb * 4u + (tid >> 6);
+    float4 v = {0.f, 0.f, 0.f, 0.f};
+    if (blk < n_blk) v = *(const float4 *)(p.x + (uint64_t)blk * 256u + lane * 4u);
+    for (; blk < n_blk; blk += step) {
+        float4 nxt = {0.f, 0.f, 0.f, 0.f};
+        if (blk + step < n_blk) nxt = *(const float4 *)(p.x + (uint64_t)(blk + step) * 256u + lane * 4u);
         const uint32_t t = blk / p.n_sb, b = blk - t * p.n_sb;
-        const float4 v = *(const float4 *)(p.x + (uint64_t)t * p.n_sb * 256u + (size_t)b * 256u + lane * 4u);
         uint8_t *row = p.xp + (uint64_t)t * p.xp_row_bytes;
         quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
+        v = nxt;
     }
 }
 
@@ -614,10 +622,18 @@ __global__ __launch_bounds__(kGbThreads) void k_group_count(
     const uint32_t n_groups = n_expert + (extra ? 1u : 0u);
     for (uint32_t e = tid; e < n_groups; e += kGbThreads) s_count[e] = 0;
     __syncthreads();
-    for (uint32_t i = tid; i < total; i += kGbThreads) {
-        const int e = selected[i];
+    auto count = [&](int e) {
         if (e >= 0 && (uint32_t)e < n_expert) atomicAdd(&s_count[e], 1);
+    };
+    const uint32_t n4 = (((uintptr_t)selected & 15u) == 0u) ? total / 4u : 0u;  // 16-byte loads
+    for (uint32_t i = tid; i < n4; i += kGbThreads) {
+        const int4 q = *(const int4 *)(selected + 4u * i);
+        count(q.x);
+        count(q.y);
+        count(q.z);
+        count(q.w);
     }
+    for (uint32_t i = 4u * n4 + tid; i < total; i += kGbThreads) count(selected[i]);
     if (extra && tid == 0) s_count[n_expert] = (int)b;
     __syncthreads();
     if (tid == 0) {
