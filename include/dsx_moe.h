@@ -273,7 +273,8 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
  * gemm_min_tokens: from this many tokens on, a layer with MXFP4 gate/up runs the grouped-GEMM
  * path (128 token columns per work item, shared expert as an extra group; a Q8_0 down matrix
- * takes the int8 grouped GEMM).
+ * takes the int8 grouped GEMM); an all-MXFP4 layer whose GEMMs use the narrow tile (below)
+ * switches at 11/16 of it.
  * decode_max_tokens: up to this many tokens, an all-MXFP4 layer runs the one-token decode
  * kernels once per token inside the same launches (no grouping by expert).
  * gemm_narrow_members: while the picks per expert average less than this, the all-MXFP4
