@@ -582,10 +582,11 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
 #pragma unroll
                     for (uint32_t mm = 0; mm < M; mm++) {
                         const v4i32 s = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[mm][b], bv, v4i32{0, 0, 0, 0}, 0, 0, 0);
-                        acc[mm][j][0] += dw[mm][0][b] * xsv[b] * (float)s.x;
-                        acc[mm][j][1] += dw[mm][1][b] * xsv[b] * (float)s.y;
-                        acc[mm][j][2] += dw[mm][2][b] * xsv[b] * (float)s.z;
-                        acc[mm][j][3] += dw[mm][3][b] * xsv[b] * (float)s.w;
+                        // three vector instructions per value: scale product, convert, fused add
+                        acc[mm][j][0] = fmaf(dw[mm][0][b] * xsv[b], (float)s.x, acc[mm][j][0]);
+                        acc[mm][j][1] = fmaf(dw[mm][1][b] * xsv[b], (float)s.y, acc[mm][j][1]);
+                        acc[mm][j][2] = fmaf(dw[mm][2][b] * xsv[b], (float)s.z, acc[mm][j][2]);
+                        acc[mm][j][3] = fmaf(dw[mm][3][b] * xsv[b], (float)s.w, acc[mm][j][3]);
                     }
                 }
             }
