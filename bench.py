@@ -300,6 +300,14 @@ def main():
         hip.l.hipEventRecord(b, stream)
     torch.cuda.synchronize()
     tiny_us = float(np.median([hip.elapsed_ms(a, b) for a, b in tiny]) * 1e3)
+    # and around nothing at all
+    empty = [(hip.event(), hip.event()) for _ in range(64)]
+    for j, (a, b) in enumerate(empty):
+        step(W + j % K)
+        hip.l.hipEventRecord(a, stream)
+        hip.l.hipEventRecord(b, stream)
+    torch.cuda.synchronize()
+    empty_us = float(np.median([hip.elapsed_ms(a, b) for a, b in empty]) * 1e3)
 
     # a copy of known size, so that byte counters collected over this run can be scaled
     from deepstrix_amd import synth
@@ -313,6 +321,7 @@ def main():
     # other token counts of the same config (informative)
     extra = {"gate_up_us_p50": float(np.median(gu_ms) * 1e3),
              "event_bracket_of_one_workgroup_kernel_us": tiny_us,
+             "event_bracket_of_nothing_us": empty_us,
              "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
              "layer_GBps_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9,
              "layer_frac_of_hbm_peak_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
