@@ -75,6 +75,7 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gemm<false, kGemmMTNarrow>);
         allow_lds(k_mxfp4_down_decode<false>);
         allow_lds(k_mxfp4_down_decode<true>);
+        allow_lds(k_mxfp4_down_decode<true, 9>);
         allow_lds(k_mxfp4_down_by_expert<1, false>);
         allow_lds(k_mxfp4_down_by_expert<2, false>);
         allow_lds(k_mxfp4_down_by_expert<4, false>);
@@ -371,7 +372,9 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     const uint32_t even = (n_rows + 2u * g_num_cu - 1u) / (2u * g_num_cu);
     p.rows_per_wg = std::min(16u, std::max(8u, even));
     const uint32_t gx = (n_rows + p.rows_per_wg - 1u) / p.rows_per_wg;
-    if (staged)
+    if (staged && units == 9u * kDownWaves)  // the V3 shape: 9 slots x 8 super-blocks, 9 units per wave
+        hipLaunchKernelGGL((k_mxfp4_down_decode<true, 9>), dim3(gx, n_tokens), dim3(kDownWaves * 64), lds, st, p);
+    else if (staged)
         hipLaunchKernelGGL(k_mxfp4_down_decode<true>, dim3(gx, n_tokens), dim3(kDownWaves * 64), lds, st, p);
     else
         hipLaunchKernelGGL(k_mxfp4_down_decode<false>, dim3(gx, n_tokens), dim3(kDownWaves * 64), lds, st, p);

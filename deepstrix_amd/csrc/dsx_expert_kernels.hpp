@@ -213,14 +213,17 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     const uint8_t *grow = gate_e + (uint64_t)(row0 + r) * row_stride;
     const uint8_t *urow = up_e + (uint64_t)(row0 + r) * row_stride;
     uint32_t sb = wave;
-    WSuper g0 = {}, u0 = {}, g1 = {}, u1 = {};
-    if (sb < p.n_blocks) {
-        g0 = load_wsuper(grow + (uint64_t)sb * kSuperBytes, kb);
-        u0 = load_wsuper(urow + (uint64_t)sb * kSuperBytes, kb);
-    }
-    if (sb + kGuWaves < p.n_blocks) {
-        g1 = load_wsuper(grow + (uint64_t)(sb + kGuWaves) * kSuperBytes, kb);
-        u1 = load_wsuper(urow + (uint64_t)(sb + kGuWaves) * kSuperBytes, kb);
+    // The first two loads are unconditional as well (a wave without a block of its own reads
+    // the row's last one and never uses it), so that the k loop starts from a known count of
+    // loads in flight.
+    WSuper g0, u0, g1, u1;
+    {
+        const uint32_t last = p.n_blocks - 1u;
+        const uint32_t b0 = sb < last ? sb : last, b1 = sb + kGuWaves < last ? sb + kGuWaves : last;
+        g0 = load_wsuper(grow + (uint64_t)b0 * kSuperBytes, kb);
+        u0 = load_wsuper(urow + (uint64_t)b0 * kSuperBytes, kb);
+        g1 = load_wsuper(grow + (uint64_t)b1 * kSuperBytes, kb);
+        u1 = load_wsuper(urow + (uint64_t)b1 * kSuperBytes, kb);
     }
 
     // ---- activations into LDS -----------------------------------------------------------
@@ -260,21 +263,46 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         mfma_super(acc_g, g, bs, yd, kb);
         mfma_super(acc_u, u, bs, yd, kb);
     };
-    while (sb < p.n_blocks) {
+    // Steady state: both refills of an iteration happen, unconditionally, so the count of loads
+    // in flight is the same on every path and each wait leaves the younger super-block's loads
+    // outstanding (behind a condition the compiler waits for everything at the join).  The empty
+    // asm statements keep each refill behind the products that read the registers it overwrites:
+    // left alone the compiler moves the refill in front of them, into fresh registers, copies
+    // those into place at the end of the iteration and waits for them there -- one super-block
+    // in flight instead of two.
+#define DSX_AFTER_PRODUCTS() asm volatile("" : "+v"(acc_g), "+v"(acc_u) :: "memory")
+#define DSX_PIN() asm volatile("" ::: "memory")
+    while (sb + 3 * kGuWaves < p.n_blocks) {
         compute(sb, g0, u0);
-        if (sb + 2 * kGuWaves < p.n_blocks) {
-            g0 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
-            u0 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
-        }
-        sb += kGuWaves;
-        if (sb >= p.n_blocks) break;
-        compute(sb, g1, u1);
-        if (sb + 2 * kGuWaves < p.n_blocks) {
-            g1 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
-            u1 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
-        }
-        sb += kGuWaves;
+        DSX_AFTER_PRODUCTS();
+        g0 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+        u0 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+        DSX_PIN();
+        // (the scale bytes of the second pair are not touched before this point either)
+        asm volatile("" : "+v"(g1.s.x), "+v"(g1.s.y), "+v"(u1.s.x), "+v"(u1.s.y));
+        compute(sb + kGuWaves, g1, u1);
+        DSX_AFTER_PRODUCTS();
+        g1 = load_wsuper(grow + (uint64_t)(sb + 3 * kGuWaves) * kSuperBytes, kb);
+        u1 = load_wsuper(urow + (uint64_t)(sb + 3 * kGuWaves) * kSuperBytes, kb);
+        DSX_PIN();
+        sb += 2 * kGuWaves;
     }
+    // Tail: up to three super-blocks are left for this wave (sb in g0/u0, sb + W in g1/u1, and
+    // sb + 2 W still to fetch, into a third pair so that it can be requested first).
+    if (sb < p.n_blocks) {
+        WSuper g2 = {}, u2 = {};
+        const bool third = sb + 2 * kGuWaves < p.n_blocks;
+        if (third) {
+            g2 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+            u2 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+        }
+        DSX_PIN();
+        compute(sb, g0, u0);
+        if (sb + kGuWaves < p.n_blocks) compute(sb + kGuWaves, g1, u1);
+        if (third) compute(sb + 2 * kGuWaves, g2, u2);
+    }
+#undef DSX_AFTER_PRODUCTS
+#undef DSX_PIN
 
     // ---- add the waves' partial sums in wave order, SwiGLU, store --------------------
     s_red[wave][0][0][lane] = acc_g.x;
@@ -354,7 +382,9 @@ struct DownDecodeParams {
 };
 
 // LDS: [n_slots * n_blocks_in] tiles of 512 bytes | yd[n_slots * n_blocks_in]
-template <bool STAGED>
+// NU > 0: every wave has exactly NU units (n_slots * n_blocks_in == NU * kDownWaves) and the k loop
+// is straight-line code; NU == 0: any shape.
+template <bool STAGED, int NU = 0>
 __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const DownDecodeParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[kDownWaves][4][64];
@@ -365,25 +395,38 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + (size_t)units * 512u);
 
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    // the wave index in a scalar register: the unit a wave works on is then uniform, and the
+    // pick that names its expert comes through the scalar cache instead of a vector load whose
+    // wait would also wait for every weight load in flight
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t row0 = blockIdx.x * p.rows_per_wg;
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    // rows of the 16-row fragment past the workgroup's share (or the matrix) load nothing
+    // rows of the 16-row fragment past the workgroup's share (or the matrix) repeat its last
+    // row: every lane loads, so no load sits behind a condition, and their sums are not stored
     const uint32_t n_live = min(p.rows_per_wg, p.n_rows - row0);
-    const bool live = r < n_live;
-    const uint64_t row_off = (uint64_t)(row0 + r) * nb * kSuperBytes;
+    const uint64_t row_off = (uint64_t)(row0 + min(r, n_live - 1u)) * nb * kSuperBytes;
     // blockIdx.y = token: its picks, its n_slots activation rows, its output row
     const int32_t *selected = p.selected + (uint64_t)blockIdx.y * p.n_used;
     const uint8_t *xq = p.xq + (uint64_t)blockIdx.y * p.n_slots * p.xq_slot_stride;
     float *out = p.out + (uint64_t)blockIdx.y * p.n_rows;
 
-    auto unit_ptr = [&](uint32_t un) -> const uint8_t * {
+    // the part of a unit's address that is the same for every lane
+    auto unit_base = [&](uint32_t un) -> const uint8_t * {
         const uint32_t slot = un / nb, b = un - slot * nb;
         const int e = (slot < p.n_used) ? selected[slot] : 0;
         const uint8_t *base = (slot < p.n_used) ? p.down + (uint64_t)(e < 0 ? 0 : e) * p.dbpe
                                                 : p.sh_down;
-        return base + row_off + (uint64_t)b * kSuperBytes;
+        return base + (uint64_t)b * kSuperBytes;
     };
+    auto unit_ptr = [&](uint32_t un) -> const uint8_t * { return unit_base(un) + row_off; };
+    // With a fixed unit count the addresses of the later units are worked out here, while the
+    // picks can still be read through the scalar cache (after the first asm statement below the
+    // compiler reads them with vector loads, and waiting for one of those waits for every
+    // weight load in flight).
+    const uint8_t *later[NU > 5 ? NU - 5 : 1];
+#pragma unroll
+    for (int i = 0; i + 5 < NU; i++) later[i] = unit_base(wave + (uint32_t)(i + 5) * kDownWaves);
 
     // The activation rows go out first when five loads per thread cover them: they need only
     // the token index, and (a wave's loads return in order) must not queue behind the weights.
@@ -393,18 +436,25 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     const bool early = STAGED && n_pieces <= 5u * kStep && units <= kStep;
     uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {}, ex4 = {};
     float early_yd = 0.0f;
+    // this thread's entry of the pick table in LDS (n_used >= 1), requested before the weights:
+    // a wave's loads return in order, so waiting for it later would wait for them as well
+    const int sel_mine = selected[min(tid, p.n_used - 1u)];
     auto piece_src = [&](uint32_t q) -> const uint8_t * {
         const uint32_t j = q / per_slot, c = q - j * per_slot;
         return xq + (uint64_t)j * p.xq_slot_stride + (size_t)c * 16u;
     };
     if (early) {
-        if (tid < n_pieces) ex0 = *(const uint4 *)piece_src(tid);
-        if (tid + kStep < n_pieces) ex1 = *(const uint4 *)piece_src(tid + kStep);
-        if (tid + 2u * kStep < n_pieces) ex2 = *(const uint4 *)piece_src(tid + 2u * kStep);
-        if (tid + 3u * kStep < n_pieces) ex3 = *(const uint4 *)piece_src(tid + 3u * kStep);
-        if (tid + 4u * kStep < n_pieces) ex4 = *(const uint4 *)piece_src(tid + 4u * kStep);
-        if (tid < units) {
-            const uint32_t j = tid / nb, bq = tid - j * nb;
+        // (indices past the end repeat the last piece: loads without a condition keep the
+        // count of loads in flight the same on every path, so later waits can be exact)
+        const uint32_t lastq = n_pieces - 1u;
+        ex0 = *(const uint4 *)piece_src(min(tid, lastq));
+        ex1 = *(const uint4 *)piece_src(min(tid + kStep, lastq));
+        ex2 = *(const uint4 *)piece_src(min(tid + 2u * kStep, lastq));
+        ex3 = *(const uint4 *)piece_src(min(tid + 3u * kStep, lastq));
+        ex4 = *(const uint4 *)piece_src(min(tid + 4u * kStep, lastq));
+        {
+            const uint32_t t = min(tid, units - 1u);
+            const uint32_t j = t / nb, bq = t - j * nb;
             early_yd = *((const float *)(xq + (uint64_t)j * p.xq_slot_stride + (size_t)nb * 512u) + bq);
         }
     }
@@ -412,13 +462,21 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     // five (slot, super-block) units of weights in flight per wave
     uint32_t un = wave;
     WSuper w0 = {}, w1 = {}, w2 = {}, w3 = {}, w4 = {};
-    if (un < units && live) w0 = load_wsuper(unit_ptr(un), kb);
-    if (un + kDownWaves < units && live) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
-    if (un + 2 * kDownWaves < units && live) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
-    if (un + 3 * kDownWaves < units && live) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
-    if (un + 4 * kDownWaves < units && live) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
+    if (NU > 0) {
+        w0 = load_wsuper(unit_ptr(un), kb);
+        if (NU > 1) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
+        if (NU > 2) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
+        if (NU > 3) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
+        if (NU > 4) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
+    } else {
+        if (un < units) w0 = load_wsuper(unit_ptr(un), kb);
+        if (un + kDownWaves < units) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
+        if (un + 2 * kDownWaves < units) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
+        if (un + 3 * kDownWaves < units) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
+        if (un + 4 * kDownWaves < units) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
+    }
 
-    if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? selected[tid] : 0;
+    if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? sel_mine : 0;
     if (early) {
         // (a slot's tiles are contiguous in LDS as they are in its row)
         if (tid < n_pieces) *(uint4 *)(tiles + (size_t)tid * 16u) = ex0;
@@ -446,19 +504,51 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
             mfma_super(acc, w, bs, s_yd[u], kb);
         }
     };
+    if (NU > 0) {
+        // Straight-line: step i multiplies unit i and refills its registers with unit i + 5.
+        // No load sits behind a condition, so each wait names exactly the loads that may stay in
+        // flight (behind a condition the compiler waits for all of them), and the empty asm
+        // statements keep each refill behind the products that read the registers it overwrites
+        // (moved in front of them it would need fresh registers, a copy and a wait for it).
+#define DSX_DOWN_STEP(I, W)                                                                  \
+    if (I < NU) {                                                                            \
+        compute(un + I * kDownWaves, W);                                                     \
+        asm volatile("" : "+v"(acc) :: "memory");                                            \
+        if (I + 5 < NU) W = load_wsuper(later[I + 5 < NU ? I : 0] + row_off, kb);            \
+        asm volatile("" ::: "memory");                                                       \
+    }
+        DSX_DOWN_STEP(0, w0)
+        DSX_DOWN_STEP(1, w1)
+        DSX_DOWN_STEP(2, w2)
+        DSX_DOWN_STEP(3, w3)
+        DSX_DOWN_STEP(4, w4)
+        DSX_DOWN_STEP(5, w0)
+        DSX_DOWN_STEP(6, w1)
+        DSX_DOWN_STEP(7, w2)
+        DSX_DOWN_STEP(8, w3)
+        DSX_DOWN_STEP(9, w4)
+        DSX_DOWN_STEP(10, w0)
+        DSX_DOWN_STEP(11, w1)
+        DSX_DOWN_STEP(12, w2)
+        DSX_DOWN_STEP(13, w3)
+        DSX_DOWN_STEP(14, w4)
+        static_assert(NU <= 15, "unrolled for at most 15 units per wave");
+#undef DSX_DOWN_STEP
+    } else {
 #define DSX_DOWN_STEP(W)                                                                     \
     compute(un, W);                                                                          \
-    if (un + 5 * kDownWaves < units && live) W = load_wsuper(unit_ptr(un + 5 * kDownWaves), kb); \
+    if (un + 5 * kDownWaves < units) W = load_wsuper(unit_ptr(un + 5 * kDownWaves), kb);     \
     un += kDownWaves;                                                                        \
     if (un >= units) break;
-    while (un < units) {
-        DSX_DOWN_STEP(w0)
-        DSX_DOWN_STEP(w1)
-        DSX_DOWN_STEP(w2)
-        DSX_DOWN_STEP(w3)
-        DSX_DOWN_STEP(w4)
-    }
+        while (un < units) {
+            DSX_DOWN_STEP(w0)
+            DSX_DOWN_STEP(w1)
+            DSX_DOWN_STEP(w2)
+            DSX_DOWN_STEP(w3)
+            DSX_DOWN_STEP(w4)
+        }
 #undef DSX_DOWN_STEP
+    }
 
     s_red[wave][0][lane] = acc.x;
     s_red[wave][1][lane] = acc.y;
