@@ -280,14 +280,15 @@ int dsx_q8_0_quantize_rows(dsx_stream_t stream, uint8_t *out, const float *x, ui
 }
 
 // ---- decode ---------------------------------------------------------------------------
-// staged != 0: xq is a staged row and (midp, counters) receive the fused quantization of mid.
+// staged != 0: xq is a staged row, midp receives the fused quantization of mid, and mid must hold
+// kMidUnwritten everywhere on entry (the front kernel of the layer writes it).
 static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint8_t *gate,
                                const uint8_t *up, const uint8_t *xq, const float *ew,
                                const int32_t *selected, const uint8_t *sh_gate,
                                const uint8_t *sh_up, float sh_clamp, uint64_t gbpe, uint64_t ubpe,
                                uint32_t n_used, float clamp, uint32_t n_rows, uint32_t n_blocks,
                                bool staged = false, uint8_t *midp = nullptr,
-                               int32_t *counters = nullptr, uint32_t n_tokens = 1) {
+                               uint32_t n_tokens = 1) {
     if (n_used == 0 && !sh_gate) return DSX_OK;
     if (!mid || !gate || !up || !xq || !ew || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: null pointer");
@@ -313,10 +314,9 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
     p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
     const uint32_t n_slots = n_used + (sh_gate ? 1u : 0u);
     if (staged) {
-        if (n_rows % 256 != 0 || !midp || !counters || !aligned(xq, 16))
+        if (n_rows % 256 != 0 || !midp || !aligned(xq, 16))
             return fail(DSX_ERR_SHAPE, "moe_gate_up_batch: fused mid quantization needs n_rows %% 256 == 0");
         p.midp = midp;
-        p.counters = counters;
         p.midp_row_bytes = staged_row_bytes(n_rows / 256);
         hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, true, true>),
                            dim3(n_rows / 16, n_slots * n_tokens), dim3(kGuWaves * 64), lds, st, p);

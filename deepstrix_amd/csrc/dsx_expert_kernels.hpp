@@ -27,6 +27,10 @@
 namespace dsx {
 
 constexpr int kGuWaves = 4;  // waves per gate/up workgroup
+// mid[] before a result has landed in it (a NaN with every bit set: no sum of products is one)
+constexpr uint32_t kMidUnwritten = 0xFFFFFFFFu;
+// rounds of the quantizing wave's wait for the other tiles of its block (about a microsecond each)
+constexpr uint32_t kMidSpinLimit = 1u << 17;
 #define DSX_MAX_SLOTS 17     // n_used <= 16 picks + the shared expert
 
 // Bytes of one staged activation row of n_sb super-blocks (16-byte aligned).
@@ -102,9 +106,8 @@ struct GateUpParams {
     const uint8_t *sh_gate;   // decode only: extra slot n_used (weight 1), or null
     const uint8_t *sh_up;
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
-    // fused quantization of mid (FUSE_MIDQ): staged rows out + arrival counters
+    // fused quantization of mid (FUSE_MIDQ): staged rows out; mid holds kMidUnwritten on entry
     uint8_t *midp;
-    int32_t *counters;     // [dest rows * n_rows / 256], zero on entry
     uint64_t gbpe, ubpe;
     uint32_t n_used, chunk;
     float clamp, sh_clamp;
@@ -125,7 +128,6 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     __shared__ int s_dest[NT];
     __shared__ float s_ew[NT];
     __shared__ uint32_t s_tok[NT];
-    __shared__ int s_last[NT];
 
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + (size_t)p.n_blocks * 512u * NT);
@@ -332,30 +334,31 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     }
 
     if (FUSE_MIDQ) {
-        // The sixteen row tiles of a 256-row block arrive in any order; the last one to
-        // arrive quantizes the block of mid into the staged format that down reads.
-        // Hand-off between workgroups (possibly on different XCDs, whose L2s are not
-        // coherent with each other): the mid values are stored write-through, each thread
-        // waits for its stores to be acknowledged, the workgroup meets at a barrier and one
-        // thread bumps the device-scope counter; the last arriver reads with loads that
-        // bypass its own L2.  No cache-wide write-back or invalidate is involved.
+        // The workgroup of a 256-row block's last row tile quantizes the block of mid into the
+        // staged format that down reads.  The sixteen tiles finish in any order, on any XCD
+        // (whose L2s are not coherent with each other), so: the mid buffer holds a bit pattern
+        // that no product can have (kMidUnwritten, written by the front kernel) wherever no
+        // result has landed yet; results are stored write-through; and the quantizing wave reads
+        // the block with loads that bypass its L2 until no lane sees the pattern any more.  The
+        // other fifteen workgroups do not wait for anything (no store acknowledgement, no
+        // counter round trip: 3 us per step at one token).  The tiles it waits for have smaller
+        // workgroup ids, so they were dispatched before it and depend on nothing; the spin is
+        // bounded all the same.
         const uint32_t nblk = p.n_rows / 256u, blk = row0 / 256u;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid < cnt) {
-            const int old = __hip_atomic_fetch_add(&p.counters[(uint32_t)s_dest[tid] * nblk + blk], 1,
-                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_last[tid] = (old == 15) ? 1 : 0;
-        }
-        __syncthreads();
+        if ((row0 & 255u) != 240u) return;  // uniform
         for (uint32_t j = wave; j < cnt; j += kGuWaves) {
-            if (!s_last[j]) continue;
             const float *src = p.mid + (uint64_t)s_dest[j] * p.n_rows + (size_t)blk * 256u + lane * 4u;
             float4 v;
-            v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (uint32_t spin = 0; spin < kMidSpinLimit; spin++) {
+                v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const bool landed = __float_as_uint(v.x) != kMidUnwritten && __float_as_uint(v.y) != kMidUnwritten &&
+                                    __float_as_uint(v.z) != kMidUnwritten && __float_as_uint(v.w) != kMidUnwritten;
+                if (__builtin_amdgcn_ballot_w64(!landed) == 0ull) break;  // wave-uniform
+                __builtin_amdgcn_s_sleep(2);
+            }
             uint8_t *row = p.midp + (uint64_t)s_dest[j] * p.midp_row_bytes;
             quantize_block_to_staged(v, lane, row + (size_t)blk * 512u,
                                      (float *)(row + (size_t)nblk * 512u) + blk);

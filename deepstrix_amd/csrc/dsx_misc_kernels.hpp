@@ -409,7 +409,7 @@ __global__ __launch_bounds__(256) void k_hetsplit_select(int32_t *__restrict__ o
 
 // Front of the layer in one launch: workgroups [0, n_tokens) route one token each (skipped
 // when routing is pinned), the rest quantize the activations into staged rows (one wave per
-// 256-element block) and clear the arrival counters of the fused mid quantization.
+// 256-element block) and mark the mid buffer of the fused mid quantization as unwritten.
 struct FrontParams {
     int32_t *selected;
     float *weights;
@@ -417,11 +417,11 @@ struct FrontParams {
     const float *bias;
     uint8_t *xp;        // staged rows out, xp_row_bytes apart
     const float *x;     // [n_tokens, k]
-    int32_t *counters;  // n_counters ints to clear (may be null)
+    uint32_t *fill;     // n_fill words to set to fill_value (may be null)
     uint32_t n_expert, n_used;
     float scale, eps;
     uint32_t mode, n_group, topk_group;
-    uint32_t n_tokens, n_sb, xp_row_bytes, n_counters, route;
+    uint32_t n_tokens, n_sb, xp_row_bytes, n_fill, fill_value, route;
 };
 
 __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParams p) {
@@ -435,8 +435,9 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
     }
     const uint32_t qb = blockIdx.x - n_route;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
-    for (uint32_t i = qb * kRouterThreads + tid; i < p.n_counters; i += (gridDim.x - n_route) * kRouterThreads)
-        p.counters[i] = 0;
+    // (n_fill is a multiple of 4 and the buffer 16-byte aligned)
+    for (uint32_t i = (qb * kRouterThreads + tid) * 4u; i < p.n_fill; i += (gridDim.x - n_route) * kRouterThreads * 4u)
+        *(uint4 *)(p.fill + i) = make_uint4(p.fill_value, p.fill_value, p.fill_value, p.fill_value);
     // one wave per 256-element block, grid-stride (many tokens: a few thousand workgroups
     // instead of one per four blocks)
     const uint32_t n_q = gridDim.x - n_route;
