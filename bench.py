@@ -31,7 +31,7 @@ COPY_BYTES = 256 << 20                    # size of the calibration copy (read 2
 # HBM bytes one gate/up launch moves, from hardware counters (two `rocprofv3 --pmc` runs of
 # this script: FETCH_SIZE, then WRITE_SIZE; summary under profiles/).  Each counter is scaled
 # by what it reads for the calibration copy below, whose traffic is known.  None = not measured.
-GATE_UP_TRAFFIC_BYTES = 144_987_136
+GATE_UP_TRAFFIC_BYTES = 145_672_443
 
 
 class Hip:
@@ -216,8 +216,8 @@ def chain_leg(H, torch, np, n_layers=8, T=2, steps=256):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--layers", type=int, default=4, help="independent layers the steps rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the T=4096 prefill leg")
