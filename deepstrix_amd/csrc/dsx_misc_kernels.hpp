@@ -435,9 +435,6 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
     }
     const uint32_t qb = blockIdx.x - n_route;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
-    // (n_fill is a multiple of 4 and the buffer 16-byte aligned)
-    for (uint32_t i = (qb * kRouterThreads + tid) * 4u; i < p.n_fill; i += (gridDim.x - n_route) * kRouterThreads * 4u)
-        *(uint4 *)(p.fill + i) = make_uint4(p.fill_value, p.fill_value, p.fill_value, p.fill_value);
     // one wave per 256-element block, grid-stride (many tokens: a few thousand workgroups
     // instead of one per four blocks)
     const uint32_t n_q = gridDim.x - n_route;
@@ -455,6 +452,11 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
         quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
         v = nxt;
     }
+    // the fill goes last: stores count like loads, so in front of the loop its stores would
+    // have to drain before the first block's elements count as arrived
+    // (n_fill is a multiple of 4 and the buffer 16-byte aligned)
+    for (uint32_t i = (qb * kRouterThreads + tid) * 4u; i < p.n_fill; i += n_q * kRouterThreads * 4u)
+        *(uint4 *)(p.fill + i) = make_uint4(p.fill_value, p.fill_value, p.fill_value, p.fill_value);
 }
 
 // Rows of f32 -> staged rows (the mid activations of the by-expert path).
