@@ -91,18 +91,24 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t g4 = lane >> 4, n16 = lane & 15u;
 
-    // Workgroups are dealt to the 8 XCDs round-robin by id, and each XCD has its own L2.  An
-    // XCD gets a contiguous range of work items; its 32 concurrent workgroups are then a few
-    // consecutive items (often column tiles of the same expert: they stream the same weights
-    // in step) times the row tiles of each (they stream the same activations).
+    // Workgroups are dealt to the 8 XCDs round-robin by id, and each XCD has its own L2.  The row
+    // tiles of a work item run on one XCD (they stream the same activations).  (A list sorted by
+    // width and dealt like cards balances better still and was slower: the widest tiles, bound
+    // by the matrix pipe, then all run at the same time, and so do the narrow ones, bound by the
+    // weight stream.)
     const uint32_t xcd = blockIdx.x & 7u, seq = blockIdx.x >> 3;
     const uint32_t n_items = (uint32_t)*p.n_work_items;   // the grid is only an upper bound
-    const uint32_t items_per_xcd = (n_items + 7u) / 8u;
     const uint32_t local = seq / p.n_row_tiles;
-    if (local >= items_per_xcd) return;
-    const uint32_t item = xcd * items_per_xcd + local;
+    // Many column tiles per expert (skewed routing, many tokens): the items are dealt to the XCDs
+    // like cards, which spreads the wide groups -- contiguous ranges of the list (it is by expert)
+    // left the busiest XCD with 17 % more column groups than the average at Zipf-skewed routing,
+    // against 8 % (layer at T=4096: -4.6 %).  About a tile per expert: contiguous ranges, so that
+    // an XCD streams one contiguous stretch of the weights (3-5 % faster then).
+    const bool deal = n_items > p.n_expert + (p.n_expert >> 1);
+    if (!deal && local >= (n_items + 7u) / 8u) return;  // uniform
+    const uint32_t item = deal ? local * 8u + xcd : xcd * ((n_items + 7u) / 8u) + local;
+    if (item >= n_items) return;  // uniform
     const uint32_t rt = seq % p.n_row_tiles;
-    if ((int)item >= *p.n_work_items) return;  // uniform: the grid is an upper bound
 
     const uint32_t wi = (uint32_t)p.work_items[item];
     const uint32_t e = wi >> 16, start = wi & 0xFFFFu;

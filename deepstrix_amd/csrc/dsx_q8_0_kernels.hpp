@@ -459,14 +459,19 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t g4 = lane >> 4, n16 = lane & 15u;
 
-    // an XCD gets a contiguous range of work items (their row tiles share the activations,
-    // neighbouring column tiles of an expert the weights, in that XCD's L2)
+    // the row tiles of a work item run on one XCD (they share the activations in its L2); the
+    // items are dealt to the XCDs like cards, which spreads the wide groups of skewed routing
     const uint32_t xcd = blockIdx.x & 7u, seq = blockIdx.x >> 3;
     const uint32_t n_items = (uint32_t)*p.n_work_items;  // the grid is only an upper bound
-    const uint32_t items_per_xcd = (n_items + 7u) / 8u;
     const uint32_t local = seq / p.n_row_tiles;
-    if (local >= items_per_xcd) return;
-    const uint32_t item = xcd * items_per_xcd + local;
+    // Many column tiles per expert (skewed routing, many tokens): the items are dealt to the XCDs
+    // like cards, which spreads the wide groups -- contiguous ranges of the list (it is by expert)
+    // left the busiest XCD with 17 % more column groups than the average at Zipf-skewed routing,
+    // against 8 % (layer at T=4096: -4.6 %).  About a tile per expert: contiguous ranges, so that
+    // an XCD streams one contiguous stretch of the weights (3-5 % faster then).
+    const bool deal = n_items > p.n_expert + (p.n_expert >> 1);
+    if (!deal && local >= (n_items + 7u) / 8u) return;  // uniform
+    const uint32_t item = deal ? local * 8u + xcd : xcd * ((n_items + 7u) / 8u) + local;
     const uint32_t rt = seq % p.n_row_tiles;
     if (item >= n_items) return;
 
