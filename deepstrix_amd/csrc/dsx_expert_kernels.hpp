@@ -133,7 +133,14 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     float *s_yd = (float *)(smem + (size_t)p.n_blocks * 512u * NT);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t row0 = blockIdx.x * 16u;
+    // Workgroup ids go round the 8 XCDs.  Decode: each XCD takes one contiguous eighth of the row
+    // tiles (a contiguous stretch of every matrix; a fraction of a microsecond per step) when an
+    // eighth is whole 256-row blocks, so that a block's last row tile still has the largest
+    // workgroup id of the block -- the fused mid quantization below relies on that.
+    const uint32_t bx = (!BY_EXPERT && (gridDim.x & 127u) == 0u)
+                            ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3)
+                            : blockIdx.x;
+    const uint32_t row0 = bx * 16u;
     const uint32_t n_sub = (BY_EXPERT && p.n_sub > 1u) ? p.n_sub : 1u;
     const uint32_t item = blockIdx.y / n_sub;
     const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;  // first member served here
@@ -403,7 +410,10 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     // pick that names its expert comes through the scalar cache instead of a vector load whose
     // wait would also wait for every weight load in flight
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t row0 = blockIdx.x * p.rows_per_wg;
+    // workgroup ids go round the 8 XCDs: each XCD takes one contiguous eighth of the row tiles
+    const uint32_t bx = (gridDim.x & 7u) == 0u ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3)
+                                                : blockIdx.x;
+    const uint32_t row0 = bx * p.rows_per_wg;
     const uint32_t r = lane & 15u, kb = lane >> 4;
     // rows of the 16-row fragment past the workgroup's share (or the matrix) repeat its last
     // row: every lane loads, so no load sits behind a condition, and their sums are not stored
