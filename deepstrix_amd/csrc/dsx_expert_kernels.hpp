@@ -133,11 +133,11 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     float *s_yd = (float *)(smem + (size_t)p.n_blocks * 512u * NT);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    // Workgroup ids go round the 8 XCDs.  Decode: each XCD takes one contiguous eighth of the row
-    // tiles (a contiguous stretch of every matrix; a fraction of a microsecond per step) when an
-    // eighth is whole 256-row blocks, so that a block's last row tile still has the largest
-    // workgroup id of the block -- the fused mid quantization below relies on that.
-    const uint32_t bx = (!BY_EXPERT && (gridDim.x & 127u) == 0u)
+    // Workgroup ids go round the 8 XCDs: each XCD takes one contiguous eighth of the row tiles (a
+    // contiguous stretch of every matrix; a fraction of a microsecond per decode step) -- with
+    // the fused mid quantization only when an eighth is whole 256-row blocks, so that a block's
+    // last row tile still has the largest workgroup id of the block, which it relies on.
+    const uint32_t bx = ((gridDim.x & (FUSE_MIDQ ? 127u : 7u)) == 0u)
                             ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3)
                             : blockIdx.x;
     const uint32_t row0 = bx * 16u;
@@ -608,7 +608,9 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     float *s_yd = (float *)(smem + (size_t)nb * 512u * NT);
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t row0 = blockIdx.x * 16u;
+    const uint32_t bx = (gridDim.x & 7u) == 0u ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3)
+                                                : blockIdx.x;  // an XCD's row tiles are contiguous
+    const uint32_t row0 = bx * 16u;
     const uint32_t n_sub = p.n_sub > 1u ? p.n_sub : 1u;
     const uint32_t item = blockIdx.y / n_sub;
     const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;
