@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -48,16 +49,25 @@ void allow_lds(K kernel) {
                               160 * 1024 - 16 * 1024);
 }
 
-// Function attributes belong to a device: raised once per device, with that device current.
+// Per-device state set up by dsx_init with that device current: function attributes belong to
+// a device.
 constexpr int kMaxDevices = 64;
-std::mutex g_attr_mutex;
-bool g_attr_done[kMaxDevices] = {};
-void raise_lds_limits() {
+std::mutex g_init_mutex;
+std::atomic<bool> g_dev_ready[kMaxDevices];
+
+// Entry points that launch kernels with raised LDS limits refuse to run before dsx_init: raising
+// the limits lazily would put API calls inside a caller's stream capture.
+int need_init(const char *who) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return;
-    std::lock_guard<std::mutex> lock(g_attr_mutex);
-    if (g_attr_done[dev]) return;
-    g_attr_done[dev] = true;
+    const hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(DSX_ERR_DEVICE, "%s: device %d out of range", who, dev);
+    if (!g_dev_ready[dev].load(std::memory_order_acquire))
+        return fail(DSX_ERR_DEVICE, "%s: call dsx_init() with device %d current first", who, dev);
+    return DSX_OK;
+}
+
+void raise_lds_limits() {
     {
         allow_lds(k_mxfp4_gate_up<1, false, false, false>);
         allow_lds(k_mxfp4_gate_up<1, false, true, true>);
@@ -187,8 +197,14 @@ int dsx_init(void) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(DSX_ERR_DEVICE, "dsx_init: device %d is %s; this library is built for gfx950",
                     dev, prop.gcnArchName);
+    if (dev < 0 || dev >= kMaxDevices) return fail(DSX_ERR_DEVICE, "dsx_init: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (g_dev_ready[dev].load(std::memory_order_acquire)) return DSX_OK;
     g_num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     raise_lds_limits();
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "dsx_init: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    g_dev_ready[dev].store(true, std::memory_order_release);
     return DSX_OK;
 }
 
@@ -306,7 +322,7 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
     const size_t lds = (size_t)n_blocks * 512 + (size_t)n_blocks * 4;
     if (lds > kLdsBudget)
         return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_batch: n_blocks=%u exceeds LDS staging", n_blocks);
-    raise_lds_limits();
+    if (int rc_init = need_init("gate_up_decode_impl")) return rc_init;
     GateUpParams p{};
     p.mid = mid; p.gate = gate; p.up = up; p.xq = xq; p.ew = ew; p.selected = selected;
     p.sh_gate = sh_gate; p.sh_up = sh_up; p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used;
@@ -361,7 +377,7 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     const size_t lds = units * 512 + units * 4;
     if (lds > kLdsBudget)
         return fail(DSX_ERR_UNSUPPORTED, "moe_down_batched: %zu (slot, block) tiles exceed LDS", units);
-    raise_lds_limits();
+    if (int rc_init = need_init("down_decode_impl")) return rc_init;
     DownDecodeParams p{};
     p.out = out; p.down = down; p.xq = xq; p.selected = selected; p.sh_down = sh_down;
     p.residual = residual;
@@ -459,7 +475,7 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     if ((uint64_t)max_work_items * n_sub > 65535u)
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: %u work items x %u sub-chunks exceed the grid",
                     max_work_items, n_sub);
-    raise_lds_limits();
+    if (int rc_init = need_init("gate_up_be_impl")) return rc_init;
     GateUpParams p{};
     p.mid = mid; p.gate = gate; p.up = up; p.xq = xq; p.ew = ew;
     p.group_count = group_count; p.group_offset = group_offset; p.members = expert_members;
@@ -531,7 +547,7 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
     if ((uint64_t)max_work_items * n_sub > 65535u)
         return fail(DSX_ERR_INVALID_ARG, "moe_down_by_expert: %u work items x %u sub-chunks exceed the grid",
                     max_work_items, n_sub);
-    raise_lds_limits();
+    if (int rc_init = need_init("down_be_impl")) return rc_init;
     DownByExpertParams p{};
     p.partials = partials; p.down = down; p.xq = xq;
     p.group_count = group_count; p.group_offset = group_offset; p.members = expert_members;
@@ -728,3 +744,4 @@ int dsx_dequant_rows(dsx_stream_t stream, int dtype, float *y, const uint8_t *ro
 }  // extern "C"
 
 #include "dsx_layer.inc"
+

@@ -63,7 +63,9 @@ typedef void *dsx_stream_t;
 
 int dsx_abi_version(void);
 const char *dsx_last_error(void);
-/* Checks that the current device is gfx950; call once per device before use. */
+/* Checks that the current device is gfx950 and raises the kernels' LDS limits on it; call once
+ * per device, with that device current, before any other entry point (they refuse to run
+ * otherwise: doing this lazily would put API calls inside a caller's stream capture). */
 int dsx_init(void);
 
 /* ---- router ---------------------------------------------------------------
