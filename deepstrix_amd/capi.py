@@ -86,6 +86,7 @@ SIGNATURES = {
     "dsx_moe_layer_workspace_bytes": (_sz, [_vp, _u32]),
     "dsx_moe_block_forward": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
     "dsx_moe_block_forward_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
+    "dsx_moe_layer_forward_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp]),
     "dsx_moe_layer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _sz, _vp, _vp, _vp, _vp]),
 }
 

@@ -49,11 +49,18 @@ void allow_lds(K kernel) {
                               160 * 1024 - 16 * 1024);
 }
 
+// Scratch of the one entry point that takes no workspace (dsx_moe_layer_forward_noalloc): a
+// fixed array in the code object instead of caller memory.  Host code never uses this name as
+// an address -- it is a host-side stand-in; dsx_init asks the runtime for each device's copy.
+constexpr size_t kStaticScratchBytes = DSX_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 // Per-device state set up by dsx_init with that device current: function attributes belong to
-// a device.
+// a device, and every device holds its own copy of `scratch` at its own address.
 constexpr int kMaxDevices = 64;
 std::mutex g_init_mutex;
 std::atomic<bool> g_dev_ready[kMaxDevices];
+void *g_scratch_ptr[kMaxDevices] = {};
 
 // Entry points that launch kernels with raised LDS limits refuse to run before dsx_init: raising
 // the limits lazily would put API calls inside a caller's stream capture.
@@ -204,6 +211,12 @@ int dsx_init(void) {
     raise_lds_limits();
     e = hipGetLastError();
     if (e != hipSuccess) return fail((int)e, "dsx_init: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+        return fail(e != hipSuccess ? (int)e : DSX_ERR_DEVICE, "dsx_init: hipGetSymbolAddress(scratch): %s",
+                    hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
     g_dev_ready[dev].store(true, std::memory_order_release);
     return DSX_OK;
 }
@@ -745,3 +758,28 @@ int dsx_dequant_rows(dsx_stream_t stream, int dtype, float *y, const uint8_t *ro
 
 #include "dsx_layer.inc"
 
+// ---- the layer for callers that cannot allocate ---------------------------------------------
+// Same sequencing and kernels as dsx_moe_layer_forward; the workspace is this device's copy of
+// the file-scope `scratch` array, whose address dsx_init resolved (g_scratch_ptr).  Nothing in
+// the workspace has to start at zero: every region is written before it is read within a call
+// (the front kernel fills `mid` with its "unwritten" pattern, the group builders zero their
+// own counters), exactly as with a caller's uninitialised workspace.
+extern "C" int dsx_moe_layer_forward_noalloc(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
+                                             const float *x, const float *logits, uint32_t n_tokens,
+                                             int32_t *selected_out, float *weights_out,
+                                             const int32_t *selected_in, const float *weights_in) {
+    if (n_tokens == 0) return DSX_OK;
+    if (!layer) return fail(DSX_ERR_INVALID_ARG, "moe_layer_forward_noalloc: null layer");
+    if (int rc_init = need_init("moe_layer_forward_noalloc")) return rc_init;
+    int dev = 0;
+    (void)hipGetDevice(&dev);  // checked by need_init
+    void *ws = g_scratch_ptr[dev];
+    const size_t need = dsx_moe_layer_workspace_bytes(layer, n_tokens);
+    if (need > kStaticScratchBytes)
+        return fail(DSX_ERR_UNSUPPORTED,
+                    "moe_layer_forward_noalloc: %u tokens need %zu B of scratch, the built-in array "
+                    "holds %zu B; use dsx_moe_layer_forward with a workspace",
+                    n_tokens, need, kStaticScratchBytes);
+    return layer_forward_impl(layer, stream, out, x, logits, n_tokens, ws, kStaticScratchBytes,
+                              selected_out, weights_out, selected_in, weights_in, nullptr);
+}

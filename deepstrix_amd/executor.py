@@ -146,6 +146,19 @@ class MoeLayer:
             return out, sel_out, w_out
         return out
 
+    def run_noalloc(self, x: torch.Tensor, logits: Optional[torch.Tensor], out: torch.Tensor,
+                    selected_in=None, weights_in=None, selected_out=None, weights_out=None):
+        """`run` through dsx_moe_layer_forward_noalloc: the library's built-in scratch array
+        instead of this object's workspace, every buffer supplied by the caller.  Refused
+        (DsxError, ERR_UNSUPPORTED) when the token count needs more scratch than the array."""
+        T = x.shape[0]
+        assert x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
+        p = lambda t: None if t is None else t.data_ptr()
+        check(lib().dsx_moe_layer_forward_noalloc(
+            self._h, torch.cuda.current_stream().cuda_stream, p(out), p(x), p(logits), T,
+            p(selected_out), p(weights_out), p(selected_in), p(weights_in)))
+        return out
+
 
 class MoeChain:
     """A stack of pre-norm residual MoE blocks run back to back on one stream, optionally

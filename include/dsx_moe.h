@@ -63,9 +63,10 @@ typedef void *dsx_stream_t;
 
 int dsx_abi_version(void);
 const char *dsx_last_error(void);
-/* Checks that the current device is gfx950 and raises the kernels' LDS limits on it; call once
- * per device, with that device current, before any other entry point (they refuse to run
- * otherwise: doing this lazily would put API calls inside a caller's stream capture). */
+/* Checks that the current device is gfx950, raises the kernels' LDS limits on it and resolves
+ * the device's copy of the built-in scratch array; call once per device, with that device
+ * current, before any other entry point (they refuse to run otherwise: doing this lazily would
+ * put API calls inside a caller's stream capture). */
 int dsx_init(void);
 
 /* ---- router ---------------------------------------------------------------
@@ -294,6 +295,22 @@ int dsx_moe_layer_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
                           const float *logits, uint32_t n_tokens, void *workspace,
                           size_t workspace_bytes, int32_t *selected_out, float *weights_out,
                           const int32_t *selected_in, const float *weights_in);
+
+/* dsx_moe_layer_forward without a workspace argument.  No counterpart in the reference: it is
+ * for callers that cannot allocate device memory at all (code under HIP graph capture that owns
+ * no buffers, tight serving loops, harnesses that forbid hipMalloc).  The scratch is a fixed
+ * DSX_NOALLOC_SCRATCH_BYTES array inside the library's code object; each device holds its own
+ * copy from the moment the library is loaded until the process ends, and dsx_init() resolves its
+ * address.  Calls whose dsx_moe_layer_workspace_bytes(layer, n_tokens) exceeds the array are
+ * refused with DSX_ERR_UNSUPPORTED (at the DeepSeek-V3 shape, 7168 x 2048 with 256 experts and top-8: up to 17 tokens).  Every call on a
+ * device shares that device's array: calls that overlap in time on one device (two streams, two
+ * layers) race; calls ordered on one stream do not.  Results are those of
+ * dsx_moe_layer_forward. */
+#define DSX_NOALLOC_SCRATCH_BYTES (8u << 20)
+int dsx_moe_layer_forward_noalloc(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
+                                  const float *x, const float *logits, uint32_t n_tokens,
+                                  int32_t *selected_out, float *weights_out,
+                                  const int32_t *selected_in, const float *weights_in);
 
 /* One pre-norm residual MoE block (the unit of BASELINE's chained-layer decode):
  *   h[t,:] += layer(RMSNorm(h[t,:]; norm_w, eps)),  router logits = router_w . RMSNorm(h[t,:])
