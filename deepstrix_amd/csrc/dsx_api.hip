@@ -12,6 +12,7 @@
 #include <new>
 
 #include "../../include/dsx_moe.h"
+#include "dsx_decode_fused.hpp"
 #include "dsx_expert_kernels.hpp"
 #include "dsx_gemm_kernels.hpp"
 #include "dsx_misc_kernels.hpp"
@@ -86,6 +87,8 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gate_up<2, true, true, false>);
         allow_lds(k_mxfp4_gate_up<4, true, true, false>);
         allow_lds(k_mxfp4_gate_up<8, true, true, false>);
+        allow_lds(k_mxfp4_decode_fused<8>);
+        allow_lds(k_mxfp4_decode_fused<0>);
         allow_lds(k_mxfp4_gemm<true, kGemmMT>);
         allow_lds(k_mxfp4_gemm<false, kGemmMT>);
         allow_lds(k_mxfp4_gemm<true, kGemmMTNarrow>);
@@ -317,7 +320,8 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
                                const uint8_t *sh_up, float sh_clamp, uint64_t gbpe, uint64_t ubpe,
                                uint32_t n_used, float clamp, uint32_t n_rows, uint32_t n_blocks,
                                bool staged = false, uint8_t *midp = nullptr,
-                               uint32_t n_tokens = 1) {
+                               uint32_t n_tokens = 1, uint32_t *status = nullptr,
+                               uint32_t spin_limit = 0) {
     if (n_used == 0 && !sh_gate) return DSX_OK;
     if (!mid || !gate || !up || !xq || !ew || !selected)
         return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_batch: null pointer");
@@ -346,6 +350,8 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
         if (n_rows % 256 != 0 || !midp || !aligned(xq, 16))
             return fail(DSX_ERR_SHAPE, "moe_gate_up_batch: fused mid quantization needs n_rows %% 256 == 0");
         p.midp = midp;
+        p.status = status;
+        p.spin_limit = spin_limit;
         p.midp_row_bytes = staged_row_bytes(n_rows / 256);
         hipLaunchKernelGGL((k_mxfp4_gate_up<1, false, true, true>),
                            dim3(n_rows / 16, n_slots * n_tokens), dim3(kGuWaves * 64), lds, st, p);

@@ -1,0 +1,468 @@
+// dsx_decode_fused.hpp -- the MXFP4 expert products of a decode step (few tokens) in ONE launch.
+//
+// The grid is a list of work items that the hardware hands to the CUs in order:
+//
+//   gate/up items  (token, slot, 16-row tile)   mid[token, slot, rows] = swiglu(gate.x, up.x) * ew
+//   down items     (token, slot, 64-row block)  partial[token, slot, rows] = down . Q8_K(mid[token, slot])
+//
+// All gate/up items come first.  A down item needs the whole mid row of its (token, slot), i.e.
+// the 128 gate/up tiles of that slot at the DeepSeek-V3 shape; it requests ALL of its weights
+// (a wave holds its 16 rows x 8 super-blocks in registers) and only then waits, so while the last
+// gate/up items drain, the slots they free fill with down items whose weights are already on
+// their way: the memory pipe sees one stream of gate, up and down weights with no kernel
+// boundary in it.  The item of a token's last slot adds the slots' partial rows in slot order (crates/v4flash-kernels/kernels/q2_k_accumulate_matvec_par.hip:724-729)
+// plus the residual and writes the output.
+//
+// Hand-off between workgroups (they may run on different XCDs, whose L2 caches are not coherent
+// with each other):
+//   * mid is pre-filled with a bit pattern no product can have (kMidUnwritten), results are
+//     stored write-through, and a consumer re-reads with loads that bypass its L2 until the
+//     pattern is gone.  Producers never wait for anything.
+//   * slot_done[token, slot] counts finished gate/up tiles, and ONE relay workgroup (the item
+//     between the gate/up and the down items) watches these counters and, when a slot is
+//     complete, raises ready[token, slot][0..kDfFan): the same flag in kDfFan separate cache
+//     lines.  A waiting down item polls one of them.  (A thousand workgroups polling one word
+//     queue up in a single memory channel and slow every load that passes through it; spread
+//     over many lines the polls cost nothing measurable.)  Counter and flags are hints that say
+//     when looking at mid is worth it; the pattern check stays the guarantee, because a producer
+//     does not order its counter update behind its stores.
+//   * partial rows are handed over the same way as mid: pre-filled with the pattern, stored
+//     write-through, and the item of the token's last slot (in grid order) re-reads the other
+//     slots' rows until the pattern is gone, then adds them in slot order to its own sums.
+// Waiting is safe because workgroups start in grid order and a gate/up item waits for nothing:
+// whatever a down item waits for is already running or finished.  Every wait is bounded all the
+// same; a wait that gives up records a code in *status and the kernel still exits.
+//
+// Decode gate/up: crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:200-229;
+// decode down:    crates/v4flash-kernels/kernels/mxfp4_matvec.hip:83-155.
+#pragma once
+
+#include "dsx_device.hpp"
+#include "dsx_expert_kernels.hpp"
+#include "dsx_quant.hpp"
+
+namespace dsx {
+
+constexpr int kDfWaves = 4;            // waves per workgroup (both item kinds)
+constexpr uint32_t kDfDownRows = 64;   // output rows of a down item: 16 per wave
+constexpr uint32_t kDfSpinLimit = 1u << 16;   // rounds of about half a microsecond
+constexpr uint32_t kDfFan = 32;        // copies of a slot's ready flag, one cache line each
+constexpr uint32_t kDfFanStride = 32;  // words between the copies (128 bytes)
+constexpr uint32_t kDfMaxTokens = 16;  // the flags are laid out for at most this many tokens
+
+struct DecodeFusedParams {
+    // gate/up
+    const uint8_t *gate, *up;        // [n_expert] experts, gbpe / ubpe apart
+    const uint8_t *sh_gate, *sh_up;  // shared expert (slot n_used) or null
+    uint64_t gbpe, ubpe;
+    const uint8_t *xq;               // [n_tokens] staged rows, xq_row_bytes apart
+    const float *ew;                 // [n_tokens, n_used]
+    const int32_t *selected;         // [n_tokens, n_used]
+    float *mid;                      // [n_tokens, n_slots, inter]; kMidUnwritten on entry
+    float clamp, sh_clamp;
+    // down
+    const uint8_t *down, *sh_down;
+    uint64_t dbpe;
+    float *partials;                 // [n_tokens, n_slots, hidden]; kMidUnwritten on entry
+    float *out;                      // [n_tokens, hidden]
+    const float *residual;           // [n_tokens, hidden] or null; may alias out
+    uint32_t *slot_done;             // [n_tokens, n_slots], zero on entry
+    uint32_t *ready;                 // [n_tokens, n_slots, kDfFan] flags kDfFanStride words apart, zero on entry
+    uint32_t poll_sleep;             // pause between two polls of a waiting down item, in units of 64 clocks
+    uint32_t *status;                // one word, zero on entry
+    uint32_t n_expert, n_used, n_slots, n_tokens;
+    uint32_t hidden, inter, n_sb, n_sb_in;   // n_sb = hidden / 256, n_sb_in = inter / 256
+    uint32_t gu_tiles, dn_blocks;            // inter / 16, hidden / 64
+    uint32_t n_gu_items;                     // n_tokens * n_slots * gu_tiles; the relay is item n_gu_items
+    uint32_t xq_row_bytes;
+    uint32_t spin_limit;
+    // measurement aid (null in normal use): 4 clock readings per item -- start, weights
+    // requested, wait over, end -- in units of the constant 100 MHz counter
+    uint64_t *trace;
+};
+
+__device__ __forceinline__ void df_stamp(const DecodeFusedParams &p, uint32_t item, uint32_t which) {
+    if (p.trace && threadIdx.x == 0) p.trace[(uint64_t)item * 4u + which] = wall_clock64();
+}
+
+// Slot order inside a token: the shared expert first (its weights need no routing result and
+// its down items are the first to be wanted), then the picks in slot order.
+__device__ __forceinline__ uint32_t df_slot_of(uint32_t order, uint32_t n_used, uint32_t n_slots) {
+    return n_slots > n_used ? (order == 0u ? n_used : order - 1u) : order;
+}
+
+// Position j of a group of n items -> the group's index space, so that the workgroups one XCD
+// receives (every eighth) cover one contiguous eighth of it.
+__device__ __forceinline__ uint32_t df_xcd_contiguous(uint32_t j, uint32_t n) {
+    return (n & 7u) == 0u ? (j & 7u) * (n >> 3) + (j >> 3) : j;
+}
+
+__device__ __forceinline__ void df_store_f32(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float df_load_f32(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- gate/up item ------------------------------------------------------------------------
+__device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint32_t item,
+                                                uint8_t *tiles, float *s_yd,
+                                                float (*s_red)[2][4][64]) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t per_token = p.n_slots * p.gu_tiles;
+    const uint32_t t = item / per_token, rem = item - t * per_token;
+    const uint32_t order = rem / p.gu_tiles, j = rem - order * p.gu_tiles;
+    const uint32_t slot = df_slot_of(order, p.n_used, p.n_slots);
+    const uint32_t row0 = df_xcd_contiguous(j, p.gu_tiles) * 16u;
+    df_stamp(p, item, 0);
+
+    // the token's staged row goes out first: it needs nothing but the token index, and (loads
+    // of a wave return in order) it must not queue behind the weights
+    const uint8_t *xrow = p.xq + (uint64_t)t * p.xq_row_bytes;
+    const uint32_t nq = p.n_sb * 32u;   // 16-byte pieces of the row's tiles
+    constexpr uint32_t kStep = kDfWaves * 64u;
+    uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {};
+    if (tid < nq) ex0 = *(const uint4 *)(xrow + (size_t)tid * 16u);
+    if (tid + kStep < nq) ex1 = *(const uint4 *)(xrow + (size_t)(tid + kStep) * 16u);
+    if (tid + 2u * kStep < nq) ex2 = *(const uint4 *)(xrow + (size_t)(tid + 2u * kStep) * 16u);
+    if (tid + 3u * kStep < nq) ex3 = *(const uint4 *)(xrow + (size_t)(tid + 3u * kStep) * 16u);
+    float early_yd = 0.0f;
+    if (tid < p.n_sb) early_yd = *((const float *)(xrow + (size_t)p.n_sb * 512u) + tid);
+
+    const uint8_t *gate_e, *up_e;
+    float clamp = p.clamp, ew = 1.0f;
+    if (slot < p.n_used) {
+        const int e = p.selected[t * p.n_used + slot];
+        if (e < 0 || (uint32_t)e >= p.n_expert) return;  // empty slot: its down items skip it too
+        gate_e = p.gate + (uint64_t)e * p.gbpe;
+        up_e = p.up + (uint64_t)e * p.ubpe;
+        ew = p.ew[t * p.n_used + slot];
+    } else {
+        gate_e = p.sh_gate;
+        up_e = p.sh_up;
+        clamp = p.sh_clamp;
+    }
+
+    const uint32_t r = lane & 15u, kb = lane >> 4;
+    const uint64_t row_stride = (uint64_t)p.n_sb * kSuperBytes;
+    const uint8_t *grow = gate_e + (uint64_t)(row0 + r) * row_stride;
+    const uint8_t *urow = up_e + (uint64_t)(row0 + r) * row_stride;
+    uint32_t sb = wave;
+    WSuper g0, u0, g1, u1;
+    {
+        const uint32_t last = p.n_sb - 1u;
+        const uint32_t b0 = sb < last ? sb : last, b1 = sb + kDfWaves < last ? sb + kDfWaves : last;
+        g0 = load_wsuper(grow + (uint64_t)b0 * kSuperBytes, kb);
+        u0 = load_wsuper(urow + (uint64_t)b0 * kSuperBytes, kb);
+        g1 = load_wsuper(grow + (uint64_t)b1 * kSuperBytes, kb);
+        u1 = load_wsuper(urow + (uint64_t)b1 * kSuperBytes, kb);
+    }
+
+    // rows longer than four pieces per thread take further passes
+    if (tid < nq) *(uint4 *)(tiles + (size_t)tid * 16u) = ex0;
+    if (tid + kStep < nq) *(uint4 *)(tiles + (size_t)(tid + kStep) * 16u) = ex1;
+    if (tid + 2u * kStep < nq) *(uint4 *)(tiles + (size_t)(tid + 2u * kStep) * 16u) = ex2;
+    if (tid + 3u * kStep < nq) *(uint4 *)(tiles + (size_t)(tid + 3u * kStep) * 16u) = ex3;
+    for (uint32_t q = tid + 4u * kStep; q < nq; q += kStep)
+        *(uint4 *)(tiles + (size_t)q * 16u) = *(const uint4 *)(xrow + (size_t)q * 16u);
+    if (tid < p.n_sb) s_yd[tid] = early_yd;
+    for (uint32_t b = tid + kStep; b < p.n_sb; b += kStep)
+        s_yd[b] = *((const float *)(xrow + (size_t)p.n_sb * 512u) + b);
+    __syncthreads();
+    df_stamp(p, item, 1);
+
+    v4f acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](uint32_t s, const WSuper &g, const WSuper &u) {
+        const BSuper bs = load_bsuper<1>(tiles + (size_t)s * 512u, kb, 0u);
+        const float yd = s_yd[s];
+        mfma_super(acc_g, g, bs, yd, kb);
+        mfma_super(acc_u, u, bs, yd, kb);
+    };
+    // Two super-blocks of gate and up in flight per wave.  Every load of the steady state is
+    // unconditional, so each wait names exactly the loads that may stay outstanding; the empty
+    // asm statements keep a refill behind the products that read the registers it overwrites.
+#define DSX_AFTER_PRODUCTS() asm volatile("" : "+v"(acc_g), "+v"(acc_u) :: "memory")
+#define DSX_PIN() asm volatile("" ::: "memory")
+    while (sb + 3 * kDfWaves < p.n_sb) {
+        compute(sb, g0, u0);
+        DSX_AFTER_PRODUCTS();
+        g0 = load_wsuper(grow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
+        u0 = load_wsuper(urow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
+        DSX_PIN();
+        asm volatile("" : "+v"(g1.s.x), "+v"(g1.s.y), "+v"(u1.s.x), "+v"(u1.s.y));
+        compute(sb + kDfWaves, g1, u1);
+        DSX_AFTER_PRODUCTS();
+        g1 = load_wsuper(grow + (uint64_t)(sb + 3 * kDfWaves) * kSuperBytes, kb);
+        u1 = load_wsuper(urow + (uint64_t)(sb + 3 * kDfWaves) * kSuperBytes, kb);
+        DSX_PIN();
+        sb += 2 * kDfWaves;
+    }
+    if (sb < p.n_sb) {
+        WSuper g2 = {}, u2 = {};
+        const bool third = sb + 2 * kDfWaves < p.n_sb;
+        if (third) {
+            g2 = load_wsuper(grow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
+            u2 = load_wsuper(urow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
+        }
+        DSX_PIN();
+        compute(sb, g0, u0);
+        if (sb + kDfWaves < p.n_sb) compute(sb + kDfWaves, g1, u1);
+        if (third) compute(sb + 2 * kDfWaves, g2, u2);
+    }
+#undef DSX_AFTER_PRODUCTS
+#undef DSX_PIN
+
+    // the waves' partial sums in wave order, SwiGLU, write-through store
+    s_red[wave][0][0][lane] = acc_g.x;
+    s_red[wave][0][1][lane] = acc_g.y;
+    s_red[wave][0][2][lane] = acc_g.z;
+    s_red[wave][0][3][lane] = acc_g.w;
+    s_red[wave][1][0][lane] = acc_u.x;
+    s_red[wave][1][1][lane] = acc_u.y;
+    s_red[wave][1][2][lane] = acc_u.z;
+    s_red[wave][1][3][lane] = acc_u.w;
+    __syncthreads();
+    if (tid < 16u) {
+        const uint32_t l = (tid >> 2) * 16u, i = tid & 3u;  // C layout: row 4*(l/16)+i, column l%16
+        float gs = 0.0f, us = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kDfWaves; w++) {
+            gs += s_red[w][0][i][l];
+            us += s_red[w][1][i][l];
+        }
+        const uint32_t ms = t * p.n_slots + slot;
+        df_store_f32(p.mid + (uint64_t)ms * p.inter + row0 + tid, swiglu_clamp(gs, us, clamp, ew));
+        // the hint; not ordered behind the stores on purpose (nobody waits here)
+        if (tid == 0)
+            __hip_atomic_fetch_add(p.slot_done + ms, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    df_stamp(p, item, 3);
+}
+
+// ---- relay item ----------------------------------------------------------------------------
+// One wave: lane l watches the counters of entries l, l + 64, ... (entry = token * n_slots +
+// slot) and the wave raises the kDfFan flags of every entry whose gate/up tiles are all done.
+__device__ __forceinline__ void df_relay_item(const DecodeFusedParams &p) {
+    if (threadIdx.x >= 64u) return;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t n = p.n_tokens * p.n_slots;
+    const uint32_t per_lane = (n + 63u) / 64u;   // at most 32 (host-checked)
+    uint32_t pending = 0u;                        // bit i: entry lane + 64 i still to be raised
+    for (uint32_t i = 0; i < per_lane; i++) {
+        const uint32_t idx = lane + 64u * i;
+        if (idx >= n) continue;
+        const uint32_t t = idx / p.n_slots, slot = idx - t * p.n_slots;
+        bool live = true;
+        if (slot < p.n_used) {
+            const int e = p.selected[t * p.n_used + slot];
+            live = e >= 0 && (uint32_t)e < p.n_expert;   // nobody waits for an empty slot
+        }
+        if (live) pending |= 1u << i;
+    }
+    for (uint32_t spin = 0; spin < p.spin_limit; spin++) {
+        if (__builtin_amdgcn_ballot_w64(pending != 0u) == 0ull) return;
+        for (uint32_t i = 0; i < per_lane; i++) {
+            const uint32_t idx = lane + 64u * i;
+            bool now = false;
+            if ((pending >> i) & 1u)
+                now = __hip_atomic_load(p.slot_done + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= p.gu_tiles;
+            if (now) pending &= ~(1u << i);
+            uint64_t m = __builtin_amdgcn_ballot_w64(now);
+            while (m) {   // uniform: the whole wave raises the flags of one finished entry
+                const uint32_t l = (uint32_t)__builtin_ctzll(m);
+                m &= m - 1ull;
+                const uint32_t entry = l + 64u * i;
+                if (lane < kDfFan)
+                    __hip_atomic_store(p.ready + ((uint64_t)entry * kDfFan + lane) * kDfFanStride, 1u,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+}
+
+// ---- down item ---------------------------------------------------------------------------
+// NSB > 0: inter / 256 == NSB, straight-line code with all NSB super-blocks of the wave's rows in
+// registers; NSB == 0: any inter, in passes of up to 8 super-blocks.
+template <int NSB>
+__device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_t item,
+                                             uint8_t *tiles, float *s_yd) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t nsb = NSB > 0 ? (uint32_t)NSB : p.n_sb_in;
+    const uint32_t per_token = p.n_slots * p.dn_blocks;
+    const uint32_t t = item / per_token, rem = item - t * per_token;
+    const uint32_t order = rem / p.dn_blocks, j = rem - order * p.dn_blocks;
+    const uint32_t slot = df_slot_of(order, p.n_used, p.n_slots);
+    const uint32_t row0 = df_xcd_contiguous(j, p.dn_blocks) * kDfDownRows + wave * 16u;
+    const uint32_t ms = t * p.n_slots + slot;
+    const uint32_t r = lane & 15u, kb = lane >> 4;
+    const uint32_t trace_id = p.n_gu_items + 1u + item;
+    df_stamp(p, trace_id, 0);
+
+    const uint8_t *down_e = p.sh_down;
+    bool live = true;
+    if (slot < p.n_used) {
+        const int e = p.selected[t * p.n_used + slot];
+        live = e >= 0 && (uint32_t)e < p.n_expert;
+        down_e = p.down + (uint64_t)(live ? e : 0) * p.dbpe;
+    }
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    if (live) {   // uniform over the workgroup
+        // The wave's share of the slot's mid row (blocks wave, wave + 4, ...) is requested first,
+        // through the caches: when the slot's gate/up tiles finished before this item started --
+        // the usual case, they come earlier in the grid -- the row is complete and nothing below
+        // waits for another workgroup.  (Blocks past the row's end repeat its last block, so
+        // that no load sits behind a condition.)
+        const float *mrow = p.mid + (uint64_t)ms * p.inter;
+        const uint32_t blk0 = min(wave, nsb - 1u), blk1 = min(wave + kDfWaves, nsb - 1u);
+        float4 mv0 = *(const float4 *)(mrow + (size_t)blk0 * 256u + lane * 4u);
+        float4 mv1 = *(const float4 *)(mrow + (size_t)blk1 * 256u + lane * 4u);
+
+        const uint8_t *wrow = down_e + (uint64_t)(row0 + r) * nsb * kSuperBytes;
+        constexpr int kHold = NSB > 0 ? NSB : 8;
+        WSuper w[kHold];
+        // everything this wave will ever read goes out now
+#pragma unroll
+        for (int b = 0; b < kHold; b++)
+            if (NSB > 0 || (uint32_t)b < nsb) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
+
+        auto landed = [](const float4 &v) {
+            return __float_as_uint(v.x) != kMidUnwritten && __float_as_uint(v.y) != kMidUnwritten &&
+                   __float_as_uint(v.z) != kMidUnwritten && __float_as_uint(v.w) != kMidUnwritten;
+        };
+        auto reload = [&](uint32_t blk) {   // bypassing the caches
+            const float *src = mrow + (size_t)blk * 256u + lane * 4u;
+            float4 v;
+            v.x = df_load_f32(src + 0);
+            v.y = df_load_f32(src + 1);
+            v.z = df_load_f32(src + 2);
+            v.w = df_load_f32(src + 3);
+            return v;
+        };
+        // a block is complete when no lane of the wave sees the pattern (wave-uniform)
+        auto wait_block = [&](float4 &v, uint32_t blk) {
+            bool flag_seen = false;
+            for (uint32_t spin = 0; __builtin_amdgcn_ballot_w64(!landed(v)) != 0ull; spin++) {
+                if (spin > p.spin_limit) {
+                    if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusMidWaitExpired);
+                    break;
+                }
+                if (!flag_seen) {
+                    // this item's copy of the slot's ready flag: one word in a line few others poll
+                    const uint32_t *flag = p.ready + ((uint64_t)ms * kDfFan + (item % kDfFan)) * kDfFanStride;
+                    uint32_t polls = 0;
+                    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u &&
+                           polls < p.spin_limit) {
+                        polls++;
+                        for (uint32_t z = 0; z < p.poll_sleep; z += 8u) __builtin_amdgcn_s_sleep(8);
+                    }
+                    flag_seen = true;
+                } else {
+                    __builtin_amdgcn_s_sleep(16);
+                }
+                v = reload(blk);
+            }
+        };
+        wait_block(mv0, blk0);
+        wait_block(mv1, blk1);
+        df_stamp(p, trace_id, 1);
+        if (wave < nsb) quantize_block_to_staged(mv0, lane, tiles + (size_t)blk0 * 512u, s_yd + blk0);
+        if (wave + kDfWaves < nsb) quantize_block_to_staged(mv1, lane, tiles + (size_t)blk1 * 512u, s_yd + blk1);
+        for (uint32_t blk = wave + 2u * kDfWaves; blk < nsb; blk += kDfWaves) {   // rows of more than 8 blocks
+            float4 v = *(const float4 *)(mrow + (size_t)blk * 256u + lane * 4u);
+            wait_block(v, blk);
+            quantize_block_to_staged(v, lane, tiles + (size_t)blk * 512u, s_yd + blk);
+        }
+        __syncthreads();
+        df_stamp(p, trace_id, 2);
+
+#pragma unroll
+        for (int b = 0; b < kHold; b++) {
+            if (NSB > 0 || (uint32_t)b < nsb) {
+                const BSuper bs = load_bsuper<1>(tiles + (size_t)b * 512u, kb, 0u);
+                mfma_super(acc, w[b], bs, s_yd[b], kb);
+            }
+        }
+        if (NSB == 0) {   // rows longer than 8 super-blocks: the rest in further passes
+            for (uint32_t b0 = 8u; b0 < nsb; b0 += 8u) {
+#pragma unroll
+                for (int b = 0; b < 8; b++)
+                    if (b0 + b < nsb) w[b] = load_wsuper(wrow + (uint64_t)(b0 + b) * kSuperBytes, kb);
+#pragma unroll
+                for (int b = 0; b < 8; b++) {
+                    if (b0 + b < nsb) {
+                        const BSuper bs = load_bsuper<1>(tiles + (size_t)(b0 + b) * 512u, kb, 0u);
+                        mfma_super(acc, w[b], bs, s_yd[b0 + b], kb);
+                    }
+                }
+            }
+        }
+    }
+
+    // The wave's 16 sums sit in column 0 of the fragment (lanes 0, 16, 32, 48, four rows each);
+    // lane r < 16 takes row r.
+    const int src_lane = (int)(16u * ((lane & 15u) >> 2));
+    const float c0 = __shfl(acc.x, src_lane, 64), c1 = __shfl(acc.y, src_lane, 64);
+    const float c2 = __shfl(acc.z, src_lane, 64), c3 = __shfl(acc.w, src_lane, 64);
+    const uint32_t ci = lane & 3u;
+    const float own = ci == 0u ? c0 : ci == 1u ? c1 : ci == 2u ? c2 : c3;
+    if (order + 1u != p.n_slots) {
+        // not the token's last item of these rows: leave the partial row (write-through, no
+        // waiting for anything) and go
+        if (lane < 16u) df_store_f32(p.partials + (uint64_t)ms * p.hidden + row0 + lane, own);
+        df_stamp(p, trace_id, 3);
+        return;
+    }
+    // The item of the last slot in grid order adds the rows up: the other slots' partial rows
+    // (pre-filled with the pattern; their items come earlier in the grid, so they are running or
+    // done) in slot order -- picks first, then the shared expert -- with its own sums taken
+    // from registers, plus the residual.
+    const float *col = p.partials + (uint64_t)t * p.n_slots * p.hidden + row0 + (lane & 15u);
+    float v[DSX_MAX_SLOTS];
+    for (uint32_t spin = 0;; spin++) {
+        bool missing = false;
+#pragma unroll
+        for (int q = 0; q < DSX_MAX_SLOTS; q++) {
+            v[q] = 0.0f;
+            if ((uint32_t)q < p.n_slots && (uint32_t)q != slot && lane < 16u)
+                v[q] = df_load_f32(col + (uint64_t)q * p.hidden);
+        }
+#pragma unroll
+        for (int q = 0; q < DSX_MAX_SLOTS; q++) missing |= __float_as_uint(v[q]) == kMidUnwritten;
+        if (__builtin_amdgcn_ballot_w64(missing) == 0ull) break;   // wave-uniform
+        if (spin > p.spin_limit) {
+            if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusPartialWaitExpired);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+    }
+    if (lane < 16u) {
+        float s = 0.0f;
+#pragma unroll
+        for (int q = 0; q < DSX_MAX_SLOTS; q++)
+            if ((uint32_t)q < p.n_slots) s += (uint32_t)q == slot ? own : v[q];
+        const uint64_t o = (uint64_t)t * p.hidden + row0 + lane;
+        if (p.residual) s += p.residual[o];
+        p.out[o] = s;
+    }
+    df_stamp(p, trace_id, 3);
+}
+
+// LDS (dynamic): max(n_sb, n_sb_in) tiles of 512 bytes | as many floats
+template <int NSB>
+__global__ __launch_bounds__(kDfWaves * 64) void k_mxfp4_decode_fused(const DecodeFusedParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[kDfWaves][2][4][64];
+    const uint32_t n_max = p.n_sb > p.n_sb_in ? p.n_sb : p.n_sb_in;
+    uint8_t *tiles = smem;
+    float *s_yd = (float *)(smem + (size_t)n_max * 512u);
+    if (blockIdx.x < p.n_gu_items)
+        df_gate_up_item(p, blockIdx.x, tiles, s_yd, s_red);
+    else if (blockIdx.x == p.n_gu_items)
+        df_relay_item(p);
+    else
+        df_down_item<NSB>(p, blockIdx.x - p.n_gu_items - 1u, tiles, s_yd);
+}
+
+}  // namespace dsx

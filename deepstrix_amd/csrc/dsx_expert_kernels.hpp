@@ -29,8 +29,15 @@ namespace dsx {
 constexpr int kGuWaves = 4;  // waves per gate/up workgroup
 // mid[] before a result has landed in it (a NaN with every bit set: no sum of products is one)
 constexpr uint32_t kMidUnwritten = 0xFFFFFFFFu;
-// rounds of the quantizing wave's wait for the other tiles of its block (about a microsecond each)
+// default bound, in rounds of about a microsecond, of the quantizing wave's wait for the other
+// tiles of its block
 constexpr uint32_t kMidSpinLimit = 1u << 17;
+// codes a kernel leaves in the layer's status word when one of its bounded waits gives up (the
+// first one wins; 0 = none did)
+constexpr uint32_t kStatusOk = 0u;
+constexpr uint32_t kStatusMidWaitExpired = 1u;      // a down item gave up waiting for mid values
+constexpr uint32_t kStatusMidqWaitExpired = 2u;     // the fused mid quantization gave up waiting for a tile
+constexpr uint32_t kStatusPartialWaitExpired = 3u;  // the slot-order sum gave up waiting for a partial row
 #define DSX_MAX_SLOTS 17     // n_used <= 16 picks + the shared expert
 
 // Bytes of one staged activation row of n_sb super-blocks (16-byte aligned).
@@ -108,6 +115,8 @@ struct GateUpParams {
     const int32_t *group_count, *group_offset, *members, *work_items, *n_work_items;
     // fused quantization of mid (FUSE_MIDQ): staged rows out; mid holds kMidUnwritten on entry
     uint8_t *midp;
+    uint32_t *status;      // FUSE_MIDQ: where an expired wait leaves its code (may be null)
+    uint32_t spin_limit;   // FUSE_MIDQ: bound of the wait in rounds (0 is read as kMidSpinLimit)
     uint64_t gbpe, ubpe;
     uint32_t n_used, chunk;
     float clamp, sh_clamp;
@@ -356,15 +365,24 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         for (uint32_t j = wave; j < cnt; j += kGuWaves) {
             const float *src = p.mid + (uint64_t)s_dest[j] * p.n_rows + (size_t)blk * 256u + lane * 4u;
             float4 v;
-            for (uint32_t spin = 0; spin < kMidSpinLimit; spin++) {
+            const uint32_t limit = p.spin_limit ? p.spin_limit : kMidSpinLimit;
+            bool complete = false;
+            for (uint32_t spin = 0; spin < limit; spin++) {
                 v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 const bool landed = __float_as_uint(v.x) != kMidUnwritten && __float_as_uint(v.y) != kMidUnwritten &&
                                     __float_as_uint(v.z) != kMidUnwritten && __float_as_uint(v.w) != kMidUnwritten;
-                if (__builtin_amdgcn_ballot_w64(!landed) == 0ull) break;  // wave-uniform
+                complete = __builtin_amdgcn_ballot_w64(!landed) == 0ull;  // wave-uniform
+                if (complete) break;
                 __builtin_amdgcn_s_sleep(2);
+            }
+            if (!complete) {
+                // gave up: a defined block (all zero, d = 0) instead of whatever was read, and a
+                // code in the status word for the host to find
+                v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (lane == 0 && p.status) atomicCAS(p.status, kStatusOk, kStatusMidqWaitExpired);
             }
             uint8_t *row = p.midp + (uint64_t)s_dest[j] * p.midp_row_bytes;
             quantize_block_to_staged(v, lane, row + (size_t)blk * 512u,

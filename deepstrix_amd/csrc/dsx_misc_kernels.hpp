@@ -417,7 +417,12 @@ struct FrontParams {
     const float *bias;
     uint8_t *xp;        // staged rows out, xp_row_bytes apart
     const float *x;     // [n_tokens, k]
+    const int32_t *sel_in;  // pinned routing (route == 0): copied to `selected`, picks outside [0, n_expert) as -1
     uint32_t *fill;     // n_fill words to set to fill_value (may be null)
+    uint32_t *fill2;    // a second region of n_fill2 words for the same value (may be null)
+    uint32_t n_fill2;
+    uint32_t *zero;     // n_zero words to clear: status word and hand-off counters (may be null)
+    uint32_t n_zero;
     uint32_t n_expert, n_used;
     float scale, eps;
     uint32_t mode, n_group, topk_group;
@@ -452,11 +457,33 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
         quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
         v = nxt;
     }
+    if (p.sel_in != nullptr)
+        for (uint32_t i = qb * kRouterThreads + tid; i < p.n_tokens * p.n_used; i += n_q * kRouterThreads) {
+            const int32_t e = p.sel_in[i];
+            p.selected[i] = (e < 0 || (uint32_t)e >= p.n_expert) ? -1 : e;
+        }
     // the fill goes last: stores count like loads, so in front of the loop its stores would
     // have to drain before the first block's elements count as arrived
     // (n_fill is a multiple of 4 and the buffer 16-byte aligned)
     for (uint32_t i = (qb * kRouterThreads + tid) * 4u; i < p.n_fill; i += n_q * kRouterThreads * 4u)
         *(uint4 *)(p.fill + i) = make_uint4(p.fill_value, p.fill_value, p.fill_value, p.fill_value);
+    for (uint32_t i = (qb * kRouterThreads + tid) * 4u; i < p.n_fill2; i += n_q * kRouterThreads * 4u)
+        *(uint4 *)(p.fill2 + i) = make_uint4(p.fill_value, p.fill_value, p.fill_value, p.fill_value);
+    for (uint32_t i = qb * kRouterThreads + tid; i < p.n_zero; i += n_q * kRouterThreads) p.zero[i] = 0u;
+}
+
+__global__ void k_zero_words(uint32_t *p, uint32_t n) {
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0u;
+}
+
+// Pinned routing as the layer uses it: picks outside [0, n_expert) become empty slots (-1).
+__global__ __launch_bounds__(256) void k_sanitize_picks(int32_t *__restrict__ out,
+                                                        const int32_t *__restrict__ in, uint32_t n,
+                                                        uint32_t n_expert) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n) return;
+    const int32_t e = in[i];
+    out[i] = (e < 0 || (uint32_t)e >= n_expert) ? -1 : e;
 }
 
 // Rows of f32 -> staged rows (the mid activations of the by-expert path).

@@ -104,6 +104,19 @@ class MoeLayer:
         check(lib().dsx_moe_layer_set_tuning(self._h, by_expert_chunk, gemm_min_tokens,
                                              decode_max_tokens, gemm_narrow_members))
 
+    def set_decode(self, fused: int = 0, spin_limit: int = 0):
+        """fused: 1 = one launch for gate/up + down (default), 2 = one launch per stage;
+        spin_limit: bound of the in-kernel waits (include/dsx_moe.h: dsx_moe_layer_set_decode)."""
+        check(lib().dsx_moe_layer_set_decode(self._h, fused, spin_limit))
+
+    def status(self, builtin_scratch: bool = False) -> int:
+        """Status word of the last forward on this layer's workspace (0 = ok); synchronizes."""
+        torch.cuda.synchronize()
+        v = C.c_uint32(0xFFFFFFFF)
+        check(lib().dsx_moe_layer_status(self._h, None if builtin_scratch else self.workspace.data_ptr(),
+                                         C.byref(v)))
+        return int(v.value)
+
     def block(self, h: torch.Tensor) -> torch.Tensor:
         """In place: h += layer(RMSNorm(h)), router logits = router_w . RMSNorm(h)
         (include/dsx_moe.h: dsx_moe_block_forward)."""

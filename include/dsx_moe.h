@@ -285,6 +285,29 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
  * stream weights then); 1 turns the narrow tile off. */
 int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
                              uint32_t decode_max_tokens, uint32_t gemm_narrow_members);
+/* Decode path of an all-MXFP4 layer (up to decode_max_tokens tokens); no counterpart in the
+ * reference.  fused: 1 = gate/up, mid quantization, down and the slot-order sum in ONE launch
+ * whose workgroups hand results to each other through device memory (the default), 2 = one
+ * launch per stage, 0 keeps the current value.  spin_limit (0 keeps): bound, in polling rounds
+ * of about half a microsecond, of every wait one workgroup does for another. */
+int dsx_moe_layer_set_decode(dsx_moe_layer *layer, uint32_t fused, uint32_t spin_limit);
+/* Measurement aid with no counterpart in the reference: a device buffer of n_items x 4 uint64
+ * that the one-launch decode path fills with clock readings (constant 100 MHz counter) per
+ * work item -- start, operands staged / weights requested, wait over, end; items in grid order:
+ * gate/up tiles, the relay, down blocks.  Ignored while n_items is smaller than the grid;
+ * NULL turns it off. */
+int dsx_moe_layer_set_trace(dsx_moe_layer *layer, uint64_t *trace, size_t n_items);
+/* Status word of the last dsx_moe_layer_forward / dsx_moe_block_forward that used `workspace`
+ * (NULL: the built-in scratch of dsx_moe_layer_forward_noalloc on the current device), copied
+ * to *host_out with a synchronous hipMemcpy: call it after synchronizing the stream, never
+ * under capture.  0 = every in-kernel hand-off completed; DSX_STATUS_* otherwise, and the
+ * output of that forward is then not to be used.  The reference has no such word because its
+ * kernels never wait for each other inside a launch. */
+#define DSX_STATUS_OK 0u
+#define DSX_STATUS_MID_WAIT_EXPIRED 1u  /* a down workgroup gave up waiting for mid values */
+#define DSX_STATUS_MIDQ_WAIT_EXPIRED 2u /* the fused mid quantization gave up waiting for a tile */
+#define DSX_STATUS_PARTIAL_WAIT_EXPIRED 3u /* the slot-order sum gave up waiting for a partial row */
+int dsx_moe_layer_status(const dsx_moe_layer *layer, const void *workspace, uint32_t *host_out);
 /* Bytes of caller-provided device scratch for up to max_tokens tokens. */
 size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
 /* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],
