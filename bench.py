@@ -28,10 +28,28 @@ TOKEN_BYTES = 9 * EXPERT_BYTES            # 8 routed + 1 shared = 210,567,168 B 
 GATE_UP_BYTES = 9 * 2 * MATRIX_BYTES      # what one gate/up launch streams at T = 1
 COPY_BYTES = 256 << 20                    # size of the calibration copy (read 256 MiB, write 256 MiB)
 
-# HBM bytes one gate/up launch moves, from hardware counters (two `rocprofv3 --pmc` runs of
-# this script: FETCH_SIZE, then WRITE_SIZE; summary under profiles/).  Each counter is scaled
-# by what it reads for the calibration copy below, whose traffic is known.  None = not measured.
-GATE_UP_TRAFFIC_BYTES = 145_672_443
+# The dominant kernel of a decode step: one launch that streams gate, up and down of the 8
+# picks and the shared expert.
+DOMINANT_KERNEL = "k_mxfp4_decode_fused<8>"
+# HBM bytes one launch of it moves come from hardware counters (two `rocprofv3 --pmc` runs of
+# this script: FETCH_SIZE, then WRITE_SIZE, each scaled by what it reads for the calibration
+# copy below, whose traffic is known).  The figure is read from the committed summary, which
+# names the kernel it was taken on; a summary for another kernel gives None (not measured).
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "moe_layer_decode_T1_cfg2_hbm_counters.txt")
+
+
+def measured_traffic(kernel: str):
+    """(bytes per launch, source) from the line `traffic_bytes_per_launch <kernel> <bytes>` of
+    the committed counter summary; (None, reason) when there is none for this kernel."""
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            for line in f:
+                parts = line.lstrip("# ").split()
+                if len(parts) >= 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == kernel:
+                    return int(parts[2]), os.path.relpath(TRAFFIC_SUMMARY, ROOT)
+    except OSError:
+        pass
+    return None, f"no counter summary for {kernel} in {os.path.relpath(TRAFFIC_SUMMARY, ROOT)}"
 
 
 class Hip:
@@ -106,7 +124,15 @@ def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
     dt = (time.perf_counter() - t0) / reps
     flops = 2.0 * T * (s.n_used + 1) * 3 * s.hidden * s.inter
     del layer
-    return {"tokens_per_s": T / dt, "ms_per_layer": dt * 1e3, "zipf_alpha": alpha,
+    # the bound of this arithmetic: every product is two FP8-rate instructions (the int8
+    # activations as two exact FP8 planes), so the useful rate tops out at half the FP8 peak
+    roof = {"bound": "mfma", "kernel": "k_mxfp4_gemm<true,128> + k_mxfp4_gemm<false,128> (whole layer, "
+            "wall clock)", "achieved": flops / dt / 1e12, "peak": FP8_MFMA_PEAK / 1e12,
+            "unit": "TFLOP/s", "frac": flops / dt / FP8_MFMA_PEAK,
+            "frac_of_two_plane_bound": 2.0 * flops / dt / FP8_MFMA_PEAK,
+            "frac_of_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK, "traffic": None,
+            "algorithmic_flop_per_launch": flops}
+    return {"roofline": roof, "tokens_per_s": T / dt, "ms_per_layer": dt * 1e3, "zipf_alpha": alpha,
             "top10pct_share": frac, "max_group": int(cnt.max()), "empty_experts": int((cnt == 0).sum()),
             "column_tiles_of_128": int(np.ceil(cnt / 128).sum()) + T // 128,
             "useful_flop": flops, "useful_TFLOPs": flops / dt / 1e12,
@@ -209,7 +235,7 @@ def chain_leg(H, torch, np, n_layers=8, T=2, steps=256):
     per_step_bytes = n_layers * T * 9 * EXPERT_BYTES
     return {"layers": n_layers, "tokens_per_step": T, "steps": steps,
             "eager_us_per_step": q(lat_e), "graph_us_per_step": q(lat_g),
-            "launches_per_step": n_layers * 4,
+            "launches_per_step": n_layers * 3,
             "graph_GBps_p50": per_step_bytes / (np.percentile(lat_g, 50) * 1e-6) / 1e9}
 
 
@@ -285,7 +311,8 @@ def main():
     gu_ms = np.array([hip.elapsed_ms(b, c) for (_, b, c, _) in evs])
     chain_ms = np.array([hip.elapsed_ms(a, d) for (a, _, _, d) in evs])
     gu_avg_us = float(gu_ms.mean() * 1e3)
-    achieved = GATE_UP_BYTES / (gu_avg_us * 1e-6) / 1e9
+    achieved = TOKEN_BYTES / (gu_avg_us * 1e-6) / 1e9
+    traffic, traffic_source = measured_traffic(DOMINANT_KERNEL)
 
     # what the bracket itself costs: the same pair of events around a one-workgroup kernel
     # (a 16-byte add, about a microsecond of kernel time in a kernel trace)
@@ -319,7 +346,10 @@ def main():
     del c_src, c_dst
 
     # other token counts of the same config (informative)
-    extra = {"gate_up_us_p50": float(np.median(gu_ms) * 1e3),
+    step_us = chain_ms * 1e3   # one decode step between two events on the launch stream
+    extra = {"dominant_kernel_us_p50": float(np.median(gu_ms) * 1e3),
+             "step_us_events": {"p10": float(np.percentile(step_us, 10)), "p50": float(np.percentile(step_us, 50)),
+                                "p90": float(np.percentile(step_us, 90))},
              "event_bracket_of_one_workgroup_kernel_us": tiny_us,
              "event_bracket_of_nothing_us": empty_us,
              "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
@@ -363,10 +393,12 @@ def main():
                                "scale 2.5, inter 2048); cold weights, steps rotate over "
                                f"{L} layers", "tokens_per_step": 1, "layers_rotated": L,
                    "algorithmic_bytes_per_token": TOKEN_BYTES},
-        "roofline": {"bound": "hbm", "kernel": "k_mxfp4_gate_up<1,false,true,true> (gate+up+SwiGLU "
-                     "+ mid quantization, 8 routed + 1 shared expert)", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": GATE_UP_TRAFFIC_BYTES,
-                     "algorithmic_bytes_per_launch": GATE_UP_BYTES, "avg_launch_us": gu_avg_us},
+        "roofline": {"bound": "hbm", "kernel": DOMINANT_KERNEL + " (gate + up + SwiGLU, mid quantization, "
+                     "down and the slot-order sum of 8 routed + 1 shared expert in one launch)",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": traffic_source,
+                     "algorithmic_bytes_per_launch": TOKEN_BYTES, "avg_launch_us": gu_avg_us},
         "extra": extra,
     }
 
@@ -374,6 +406,7 @@ def main():
         # CPU baseline: the oracle (a port of the reference arithmetic) on the host cores,
         # same layer-0 weights, decode tokens one at a time, bounded by --cpu-seconds.
         from oracle import ref
+        cpu_flags = ref.use_timing_build()
         dw = weights[0]
         hw = ref.MoeWeights(base.hidden, base.inter, base.n_expert, base.n_used,
                             dw.gate.cpu().numpy(), dw.up.cpu().numpy(), dw.down.cpu().numpy(),
@@ -396,7 +429,8 @@ def main():
             "value": cpu_s * 1e6 / max(done, 1), "unit": "us/token", "cores": threads,
             "kind": "port",
             "sample": f"{done} tokens decoded one at a time through the C oracle "
-                      f"(OpenMP, {threads} threads) on layer 0 of the same workload, {cpu_s:.1f} s"}
+                      f"(gcc {cpu_flags}, OpenMP, {threads} threads) on layer 0 of the same workload, "
+                      f"{cpu_s:.1f} s"}
     print(json.dumps(result))
 
 

@@ -33,6 +33,28 @@ def build(force: bool = False) -> str:
     return _SO
 
 
+def use_timing_build() -> str:
+    """For the timed CPU-baseline leg only: compiles the oracle for the host it runs on
+    (-O3 -march=native, same floating-point rules, so the same results) into a temporary
+    directory and switches this module to it.  Returns the flags in use; when the compile fails
+    the committed portable build stays in place and its flags are returned."""
+    global _lib
+    import tempfile
+    portable = "-O2 -fopenmp -ffp-contract=off -fno-fast-math"
+    flags = "-O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math"
+    try:
+        out = os.path.join(tempfile.mkdtemp(prefix="dsx_oracle_"), "libdsx_oracle_native.so")
+        subprocess.check_call(["gcc", *flags.split(), "-fPIC", "-std=c11", "-shared", "-o", out,
+                               os.path.join(_DIR, "dsx_oracle.c"), "-lm"],
+                              stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        l = C.CDLL(out)
+        _declare(l)
+        _lib = l
+        return flags
+    except (OSError, subprocess.CalledProcessError):
+        return portable
+
+
 _lib = None
 
 
