@@ -66,6 +66,7 @@ struct DecodeFusedParams {
     float *partials;                 // [n_tokens, n_slots, hidden]; kMidUnwritten on entry
     float *out;                      // [n_tokens, hidden]
     const float *residual;           // [n_tokens, hidden] or null; may alias out
+    const float *shared_rows;        // [n_tokens, hidden] or null: a shared expert computed elsewhere
     uint32_t *slot_done;             // [n_tokens, n_slots], zero on entry
     uint32_t *ready;                 // [n_tokens, n_slots, kDfFan] flags kDfFanStride words apart, zero on entry
     uint32_t poll_sleep;             // pause between two polls of a waiting down item, in units of 64 clocks
@@ -443,6 +444,7 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
         for (int q = 0; q < DSX_MAX_SLOTS; q++)
             if ((uint32_t)q < p.n_slots) s += (uint32_t)q == slot ? own : v[q];
         const uint64_t o = (uint64_t)t * p.hidden + row0 + lane;
+        if (p.shared_rows) s += p.shared_rows[o];
         if (p.residual) s += p.residual[o];
         p.out[o] = s;
     }

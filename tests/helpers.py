@@ -24,6 +24,7 @@ class Shape:
     shared: bool = True
     sh_gate_fmt: Optional[int] = None
     sh_down_fmt: Optional[int] = None
+    sh_inter: Optional[int] = None   # the shared expert's intermediate size (None: like the routed experts)
     clamp: float = 0.0
     router_mode: int = 1
     n_group: int = 1
@@ -40,6 +41,10 @@ class Shape:
     @property
     def shd(self):
         return self.sh_down_fmt if self.sh_down_fmt is not None else self.down_fmt
+
+    @property
+    def shi(self):
+        return self.sh_inter if self.sh_inter is not None else self.inter
 
 
 # BASELINE configs
@@ -69,10 +74,10 @@ def host_weights(s: Shape, experts=None) -> ref.MoeWeights:
     w = ref.MoeWeights(s.hidden, s.inter, s.n_expert, s.n_used, gate, up, down, s.gate_fmt,
                        s.gate_fmt, s.down_fmt, s.clamp)
     if s.shared:
-        w.sh_inter = s.inter
-        w.sh_gate = host_expert(s, synth.T_SH_GATE, s.shg, s.inter, s.hidden, 0)
-        w.sh_up = host_expert(s, synth.T_SH_UP, s.shg, s.inter, s.hidden, 0)
-        w.sh_down = host_expert(s, synth.T_SH_DOWN, s.shd, s.hidden, s.inter, 0)
+        w.sh_inter = s.shi
+        w.sh_gate = host_expert(s, synth.T_SH_GATE, s.shg, s.shi, s.hidden, 0)
+        w.sh_up = host_expert(s, synth.T_SH_UP, s.shg, s.shi, s.hidden, 0)
+        w.sh_down = host_expert(s, synth.T_SH_DOWN, s.shd, s.hidden, s.shi, 0)
         w.sh_gate_fmt = w.sh_up_fmt = s.shg
         w.sh_down_fmt = s.shd
         w.sh_clamp = s.clamp
@@ -103,10 +108,10 @@ def device_weights(s: Shape, device="cuda", block=False):
     if s.bias_sigma:
         w.bias = synth.normal_dev(s.seed, synth.T_BIAS, s.n_expert, s.bias_sigma)
     if s.shared:
-        w.sh_inter = s.inter
-        w.sh_gate = synth.weights_dev(s.shg, s.seed, synth.T_SH_GATE, s.inter, s.hidden)
-        w.sh_up = synth.weights_dev(s.shg, s.seed, synth.T_SH_UP, s.inter, s.hidden)
-        w.sh_down = synth.weights_dev(s.shd, s.seed, synth.T_SH_DOWN, s.hidden, s.inter)
+        w.sh_inter = s.shi
+        w.sh_gate = synth.weights_dev(s.shg, s.seed, synth.T_SH_GATE, s.shi, s.hidden)
+        w.sh_up = synth.weights_dev(s.shg, s.seed, synth.T_SH_UP, s.shi, s.hidden)
+        w.sh_down = synth.weights_dev(s.shd, s.seed, synth.T_SH_DOWN, s.hidden, s.shi)
         w.sh_gate_fmt = w.sh_up_fmt = s.shg
         w.sh_down_fmt = s.shd
         w.sh_clamp = s.clamp
@@ -129,6 +134,51 @@ def host_block_params(s: Shape):
 def oracle_route(s: Shape, logits, bias):
     return ref.router_topk(logits, bias, s.n_used, s.route_scale, s.route_eps, s.router_mode,
                            s.n_group, s.topk_group)
+
+
+def host_weights_from_device(s: Shape, dw) -> ref.MoeWeights:
+    """The layer's bytes copied back from the GPU: the cheap way to a host copy of a full-size
+    layer (the device generator makes the same bytes as the host one, which the generator tests
+    check on smaller tensors)."""
+    n = lambda t: t.cpu().numpy()
+    w = ref.MoeWeights(s.hidden, s.inter, s.n_expert, s.n_used, n(dw.gate), n(dw.up), n(dw.down),
+                       s.gate_fmt, s.gate_fmt, s.down_fmt, s.clamp)
+    if s.shared:
+        w.sh_inter = s.shi
+        w.sh_gate, w.sh_up, w.sh_down = n(dw.sh_gate), n(dw.sh_up), n(dw.sh_down)
+        w.sh_gate_fmt = w.sh_up_fmt = s.shg
+        w.sh_down_fmt = s.shd
+        w.sh_clamp = s.clamp
+    return w
+
+
+def compare_stats(a: np.ndarray, b_ref: np.ndarray) -> dict:
+    """The reference harness's comparison (scratch/kernel_ideas/_infra/kbench.h:249-270):
+    count of elements whose bits differ, max_abs, max_rel (elementwise, over elements that are
+    not tiny), rmse / ref_rms -- plus the parity metric max|a - ref| / max|ref|."""
+    a32, r32 = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b_ref, np.float32)
+    a64, r64 = a32.astype(np.float64), r32.astype(np.float64)
+    d = np.abs(a64 - r64)
+    ref_max = float(np.abs(r64).max())
+    big = np.abs(r64) > 1e-3 * max(ref_max, 1e-30)
+    return {"bit_diffs": int((a32.view(np.uint32) != r32.view(np.uint32)).sum()),
+            "max_abs": float(d.max()),
+            "max_rel": float((d[big] / np.abs(r64[big])).max()) if big.any() else 0.0,
+            "rel_rmse": float(np.sqrt((d ** 2).mean()) / max(np.sqrt((r64 ** 2).mean()), 1e-30)),
+            "max_over_max": float(d.max()) / max(ref_max, 1e-30)}
+
+
+def assert_close(a: np.ndarray, b_ref: np.ndarray, rel: float = 2e-3, what: str = "") -> dict:
+    """Parity of an output with the oracle's: the contract max|a - ref| / max|ref| < rel, and
+    elementwise |a - ref| <= rel * |ref| + floor with floor = rel * rms(ref) (an element near a
+    zero crossing is measured against the size of its neighbours, not against itself)."""
+    st = compare_stats(a, b_ref)
+    r64 = np.asarray(b_ref, np.float64)
+    floor = rel * float(np.sqrt((r64 ** 2).mean()))
+    bad = np.abs(np.asarray(a, np.float64) - r64) > rel * np.abs(r64) + floor
+    assert st["max_over_max"] < rel, f"{what}: {st}"
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than {rel} * |ref| + {floor:.3e}: {st}"
+    return st
 
 
 def max_rel(a: np.ndarray, b_ref: np.ndarray) -> float:
