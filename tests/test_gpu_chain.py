@@ -15,8 +15,9 @@ pytestmark = pytest.mark.gpu
 OUT_TOL = 2e-3
 
 
-def oracle_block(s, h, experts_cache=None):
-    """h + layer(RMSNorm(h)) on the CPU; also the smallest k/(k+1) score gap per token."""
+def oracle_block(s, h, dw=None):
+    """h + layer(RMSNorm(h)) on the CPU; also the smallest k/(k+1) score gap per token.
+    dw: the layer's device tensors, to copy the picked experts from instead of generating them."""
     norm_w, router_w = H.host_block_params(s)
     xn = ref.rms_norm(h, norm_w, 1e-6)
     logits = ref.router_logits(router_w, xn)
@@ -29,9 +30,32 @@ def oracle_block(s, h, experts_cache=None):
     for t in range(h.shape[0]):
         sc = np.sort(scores[t][np.isfinite(scores[t])])[::-1]
         gaps.append(float(sc[s.n_used - 1] - sc[s.n_used]))
-    hw = H.host_weights(s, experts=np.unique(sel))
+    hw = (H.host_weights(s, experts=np.unique(sel)) if dw is None
+          else H.host_weights_from_device(s, dw, experts=np.unique(sel)))
     out = ref.moe_forward(hw, xn, sel, w)
     return (h + out).astype(np.float32), xn, logits, np.array(gaps)
+
+
+def verify_chain_stepwise(chain, shapes, h, tol, min_checked):
+    """Every block of the chain on the chain's OWN running state against the oracle on that same
+    state: rows whose k-th / (k+1)-th routing scores are further apart than 1e-4 must agree
+    (the layer's contribution within `tol`), and at least `min_checked` rows must be such rows.
+    Returns the state after the last block, which one `chain.step` must reproduce bit for bit --
+    so the end-to-end result is checked whatever the routing margins are."""
+    cur = np.array(h, np.float32)
+    checked = 0
+    for i, s in enumerate(shapes):
+        want, _, _, gaps = oracle_block(s, cur, chain.layers[i].w)
+        dh = torch.from_numpy(cur).cuda()
+        chain.layers[i].block(dh)
+        got = dh.cpu().numpy()
+        ok = gaps > 1e-4
+        if ok.any():
+            assert H.max_rel(got[ok] - cur[ok], want[ok] - cur[ok]) < tol, f"layer {i}"
+            checked += int(ok.sum())
+        cur = got
+    assert checked >= min_checked, f"only {checked} rows had a routing margin above 1e-4"
+    return cur
 
 
 def layer_shapes(base, n):
@@ -103,14 +127,6 @@ def test_block_matches_oracle(T):
     assert H.max_rel(got[ok], want[ok]) < OUT_TOL
 
 
-def run_chain_oracle(shapes, h):
-    min_gap = np.inf
-    for s in shapes:
-        h, _, _, gaps = oracle_block(s, h)
-        min_gap = min(min_gap, gaps.min())
-    return h, min_gap
-
-
 def test_small_chain_eager_and_graph():
     base = H.Shape(512, 256, 8, 2, router_mode=1, route_scale=2.5, clamp=10.0, seed=111)
     shapes = layer_shapes(base, 3)
@@ -119,14 +135,15 @@ def test_small_chain_eager_and_graph():
     chain.capture(2)
     for step in range(4):   # fresh inputs each step; eager work between the replays
         h = rng.normal(0, 1, (2, base.hidden)).astype(np.float32)
-        want, min_gap = run_chain_oracle(shapes, h)
         eager = chain.step(torch.from_numpy(h).cuda()).clone()
         torch.cuda.synchronize()
         replayed = chain.replay(torch.from_numpy(h).cuda()).clone()
         torch.cuda.synchronize()
         assert torch.equal(eager, replayed), f"graph replay {step} differs from the eager step"
-        if min_gap > 1e-2:   # every pick decided by a margin far above the f32 noise carried along
-            assert H.max_rel(eager.cpu().numpy(), want) < 3 * OUT_TOL   # three layers deep
+        # hidden = 512: one rounding step of an activation weighs several times what it does at
+        # the real width, hence the wider bar (see test_block_matches_oracle)
+        final = verify_chain_stepwise(chain, shapes, h, 3 * OUT_TOL, min_checked=5)
+        assert np.array_equal(final, eager.cpu().numpy())
 
 
 @pytest.mark.parametrize("T,fmt", [(16, "mxfp4"), (130, "mxfp4"), (16, "q8_0"), (130, "q8_0"), (130, "mixed")])
@@ -152,9 +169,8 @@ def test_graph_replay_of_the_by_expert_and_gemm_paths(T, fmt):
         replayed = chain.replay(torch.from_numpy(h).cuda()).clone()
         torch.cuda.synchronize()
         assert torch.equal(eager, replayed), f"graph replay {step} differs from the eager step"
-    want, min_gap = run_chain_oracle(shapes, h)
-    if min_gap > 1e-2:
-        assert H.max_rel(eager.cpu().numpy(), want) < 3 * OUT_TOL
+    final = verify_chain_stepwise(chain, shapes, h, 3 * OUT_TOL, min_checked=(9 * 2 * T) // 10)
+    assert np.array_equal(final, eager.cpu().numpy())
 
 
 def test_config4_chain_of_v3_layers():
@@ -163,28 +179,15 @@ def test_config4_chain_of_v3_layers():
     chain = MoeChain([H.device_weights(s, block=True) for s in shapes], 2)
     rng = np.random.default_rng(4)
     h = rng.normal(0, 1, (2, H.CFG2.hidden)).astype(np.float32)
-    # layer by layer on the oracle's running state, so that one near-tie cannot hide the rest
-    cur = h
-    checked = 0
-    for i, s in enumerate(shapes):
-        want, _, _, gaps = oracle_block(s, cur)
-        dh = torch.from_numpy(cur).cuda()
-        chain.layers[i].block(dh)
-        got = dh.cpu().numpy()
-        ok = gaps > 1e-4
-        if ok.any():
-            assert H.max_rel(got[ok] - cur[ok], want[ok] - cur[ok]) < OUT_TOL, f"layer {i}"
-            checked += int(ok.sum())
-        cur = want
-    assert checked >= 12
+    # layer by layer on the chain's own running state: each block is checked against the oracle
+    # on the very input the GPU chain feeds it, so the end-to-end state is verified transitively
+    final = verify_chain_stepwise(chain, shapes, h, OUT_TOL, min_checked=12)
     chain.capture(2)
     eager = chain.step(torch.from_numpy(h).cuda()).clone()
     for _ in range(3):
         replayed = chain.replay(torch.from_numpy(h).cuda()).clone()
         torch.cuda.synchronize()
         assert torch.equal(eager, replayed)
-    # End to end the state carries each layer's f32-level differences into the next router, so
-    # the whole chain is only comparable when every pick is decided by a comfortable margin.
-    want_all, min_gap = run_chain_oracle(shapes, h)
-    if min_gap > 1e-2:
-        assert H.max_rel(eager.cpu().numpy(), want_all) < 8 * OUT_TOL
+    assert np.array_equal(final, eager.cpu().numpy())
+    for layer in chain.layers:
+        assert layer.status() == 0
