@@ -617,6 +617,7 @@ int dsx_moe_reduce_partials(dsx_stream_t stream, float *out, const float *partia
 
 extern "C++" {
 namespace {
+constexpr uint32_t kRouterTiledMinTokens = 16;  // from here on the router matvec runs as a tiled GEMM
 template <typename WT>
 int router_logits_impl(dsx_stream_t stream, float *logits, const WT *router_w, const float *x,
                        uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
@@ -625,6 +626,12 @@ int router_logits_impl(dsx_stream_t stream, float *logits, const WT *router_w, c
     if (n_expert == 0 || hidden == 0) return fail(DSX_ERR_INVALID_ARG, "router_logits: n_expert=%u hidden=%u", n_expert, hidden);
     if (!aligned(router_w, 16) || !aligned(x, 16))
         return fail(DSX_ERR_SHAPE, "router_logits: router_w and x must be 16-byte aligned");
+    if (n_tokens >= kRouterTiledMinTokens && hidden % 16 == 0 && n_expert % 4 == 0 && aligned(logits, 16)) {
+        // many tokens: tiles of 32 experts x 32 tokens on the f32 matrix instruction
+        hipLaunchKernelGGL((k_router_logits_tiled<WT>), dim3((n_expert + 31) / 32, (n_tokens + 31) / 32),
+                           dim3(256), 0, S(stream), logits, router_w, x, n_expert, hidden, n_tokens);
+        return launched("router_logits");
+    }
     hipLaunchKernelGGL((k_router_logits<false, WT>), dim3(n_expert), dim3(256), 0, S(stream), logits,
                        (float *)nullptr, router_w, x, (const float *)nullptr, 0.0f, n_expert, hidden,
                        n_tokens);

@@ -827,14 +827,19 @@ __global__ __launch_bounds__(256) void k_swiglu_clamp_weighted(float *__restrict
     mid[idx] = swiglu_clamp(gate[idx], up[idx], clamp, expert_w[e]);
 }
 
-// RMS norm, one workgroup per row: 256 strided f64 partial sums, f32 tree, then scale.
-// crates/v4flash-kernels/kernels/rms_norm.hip:12-50
+// RMS norm, one workgroup per row: 256 strided f64 partial sums, rounded to f32 and added up in
+// the order of the reference's tree (element t takes t + 128, then t + 64, ... t + 1:
+// crates/v4flash-kernels/kernels/rms_norm.hip:12-50), then the scale.  The order is the parity
+// contract; how it is carried out is not: the 256 values cross the four waves once through LDS
+// (strides 128 and 64 are lane-wise sums of whole waves) and the last six steps are shifts
+// inside wave 0, so there are two barriers instead of eight.
 __global__ __launch_bounds__(256) void k_rms_norm(float *__restrict__ out,
                                                   const float *__restrict__ x,
                                                   const float *__restrict__ weight, uint32_t n,
                                                   float eps) {
-    __shared__ float sdata[256];
-    const uint32_t tid = threadIdx.x;
+    __shared__ float s_part[4][64];
+    __shared__ float s_total;
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const float *xr = x + (uint64_t)blockIdx.x * n;
     float *orow = out + (uint64_t)blockIdx.x * n;
     double partial = 0.0;
@@ -842,13 +847,18 @@ __global__ __launch_bounds__(256) void k_rms_norm(float *__restrict__ out,
         const float v = xr[i];
         partial += (double)v * (double)v;
     }
-    sdata[tid] = (float)partial;
+    s_part[wave][lane] = (float)partial;
     __syncthreads();
-    for (uint32_t stride = 128; stride > 0; stride >>= 1) {
-        if (tid < stride) sdata[tid] += sdata[tid + stride];
-        __syncthreads();
+    if (wave == 0u) {
+        const float a = s_part[0][lane] + s_part[2][lane];   // stride 128, elements 0..63
+        const float b = s_part[1][lane] + s_part[3][lane];   // stride 128, elements 64..127
+        float c = a + b;                                      // stride 64
+#pragma unroll
+        for (int stride = 32; stride > 0; stride >>= 1) c += __shfl_down(c, stride, 64);
+        if (lane == 0u) s_total = c;
     }
-    const float mean_sq = sdata[0] / (float)n;
+    __syncthreads();
+    const float mean_sq = s_total / (float)n;
     const float scale = 1.0f / sqrtf(mean_sq + eps);
     for (uint32_t i = tid; i < n; i += 256u) orow[i] = xr[i] * scale * weight[i];
 }
@@ -1181,6 +1191,43 @@ __global__ __launch_bounds__(256) void k_q8_0_repack_rows(uint8_t *__restrict__ 
 }
 
 // Identity grouping for a dense expert: every token is a member of expert 0 with weight 1.
+// Router logits for many tokens: logits[t, e] = sum_k W[e, k] * x[t, k] with f32 products and
+// sums on the f32 matrix instruction (v_mfma_f32_16x16x4_f32).  A workgroup of four waves
+// computes 32 experts x 32 tokens, one 16 x 16 fragment per wave; a lane fetches four consecutive
+// k of its row of W and of its row of x with one 128-bit load each and feeds them to four
+// instructions (k is summed over, so any assignment of k to instructions is the same sum up to
+// f32 order).  Every operand row is read once per tile instead of once per expert.
+// hidden % 16 == 0, n_expert % 4 == 0.
+// (crates/v4flash-kernels/src/het/forward_prefill.rs:8974-9015, the engine's batched router GEMM.)
+typedef float v4f_rl __attribute__((ext_vector_type(4)));
+template <typename WT>
+__global__ __launch_bounds__(256) void k_router_logits_tiled(float *__restrict__ logits,
+                                                             const WT *__restrict__ w,
+                                                             const float *__restrict__ x,
+                                                             uint32_t n_expert, uint32_t hidden,
+                                                             uint32_t n_tokens) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t e0 = blockIdx.x * 32u + (wave & 1u) * 16u, t0 = blockIdx.y * 32u + (wave >> 1) * 16u;
+    if (e0 >= n_expert || t0 >= n_tokens) return;  // uniform per wave; no barrier below
+    const uint32_t r = lane & 15u, kg = lane >> 4;
+    // rows past the end repeat the last one (loaded, never stored)
+    const WT *wr = w + (uint64_t)min(e0 + r, n_expert - 1u) * hidden + 4u * kg;
+    const float *xr = x + (uint64_t)min(t0 + r, n_tokens - 1u) * hidden + 4u * kg;
+    v4f_rl acc = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t k = 0; k < hidden; k += 16u) {
+        const float4 a = router_w4(wr + k);
+        const float4 b = *(const float4 *)(xr + k);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc, 0, 0, 0);
+    }
+    // the lane holds experts e0 + 4 kg .. + 3 of token t0 + r
+    const uint32_t t = t0 + r, e = e0 + 4u * kg;
+    if (t < n_tokens && e < n_expert)
+        *(float4 *)(logits + (uint64_t)t * n_expert + e) = make_float4(acc.x, acc.y, acc.z, acc.w);
+}
+
 __global__ __launch_bounds__(256) void k_dense_groups(int32_t *__restrict__ group_count,
                                                       int32_t *__restrict__ group_offset,
                                                       int32_t *__restrict__ members,

@@ -64,7 +64,11 @@ def layer_shapes(base, n):
 
 def test_router_logits_operator():
     rng = np.random.default_rng(0)
-    for T, E, hidden in [(1, 64, 2048), (5, 256, 7168), (9, 16, 520), (3, 7, 30), (2, 5, 1026)]:
+    # from 16 tokens on (hidden % 16 == 0, E % 4 == 0) the matvec runs as a tiled GEMM on the f32
+    # matrix instruction: full tiles, ragged tiles in both directions, and shapes that fall back
+    for T, E, hidden in [(1, 64, 2048), (5, 256, 7168), (9, 16, 520), (3, 7, 30), (2, 5, 1026),
+                         (16, 32, 64), (40, 256, 7168), (130, 384, 5120), (33, 20, 48), (17, 7, 64),
+                         (64, 64, 1030)]:
         W = rng.normal(0, 0.02, (E, hidden)).astype(np.float32)
         x = rng.normal(0, 1, (T, hidden)).astype(np.float32)
         out = torch.zeros((T, E), dtype=torch.float32, device="cuda")
@@ -76,7 +80,8 @@ def test_router_logits_operator_f16_weights():
     """The engine keeps the router matrix in f16 (crates/v4flash-kernels/src/f16.rs:37-45):
     products and sums stay f32, so the result equals the f32 matvec over the widened weights."""
     rng = np.random.default_rng(1)
-    for T, E, hidden in [(1, 384, 5120), (5, 256, 7168), (9, 16, 520), (3, 7, 30), (2, 5, 1026)]:
+    for T, E, hidden in [(1, 384, 5120), (5, 256, 7168), (9, 16, 520), (3, 7, 30), (2, 5, 1026),
+                         (40, 256, 7168), (33, 20, 48)]:
         W16 = rng.normal(0, 0.02, (E, hidden)).astype(np.float16)
         x = rng.normal(0, 1, (T, hidden)).astype(np.float32)
         out = torch.zeros((T, E), dtype=torch.float32, device="cuda")
