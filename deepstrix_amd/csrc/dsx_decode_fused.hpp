@@ -69,6 +69,7 @@ struct DecodeFusedParams {
     const float *shared_rows;        // [n_tokens, hidden] or null: a shared expert computed elsewhere
     uint32_t *slot_done;             // [n_tokens, n_slots], zero on entry
     uint32_t *ready;                 // [n_tokens, n_slots, kDfFan] flags kDfFanStride words apart, zero on entry
+    uint32_t dn_early;               // super-blocks of a down item's weights requested before its mid row is checked
     uint32_t poll_sleep;             // pause between two polls of a waiting down item, in units of 64 clocks
     uint32_t *status;                // one word, zero on entry
     uint32_t n_expert, n_used, n_slots, n_tokens;
@@ -323,10 +324,12 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
         const uint8_t *wrow = down_e + (uint64_t)(row0 + r) * nsb * kSuperBytes;
         constexpr int kHold = NSB > 0 ? NSB : 8;
         WSuper w[kHold];
-        // everything this wave will ever read goes out now
+        // the first part of what this wave will read goes out now, the rest once the mid row is
+        // known to be there
+        const int early = (int)p.dn_early;
 #pragma unroll
         for (int b = 0; b < kHold; b++)
-            if (NSB > 0 || (uint32_t)b < nsb) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
+            if ((NSB > 0 || (uint32_t)b < nsb) && b < early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
 
         auto landed = [](const float4 &v) {
             return __float_as_uint(v.x) != kMidUnwritten && __float_as_uint(v.y) != kMidUnwritten &&
@@ -367,6 +370,9 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
         };
         wait_block(mv0, blk0);
         wait_block(mv1, blk1);
+#pragma unroll
+        for (int b = 0; b < kHold; b++)
+            if ((NSB > 0 || (uint32_t)b < nsb) && b >= early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
         df_stamp(p, trace_id, 1);
         if (wave < nsb) quantize_block_to_staged(mv0, lane, tiles + (size_t)blk0 * 512u, s_yd + blk0);
         if (wave + kDfWaves < nsb) quantize_block_to_staged(mv1, lane, tiles + (size_t)blk1 * 512u, s_yd + blk1);
