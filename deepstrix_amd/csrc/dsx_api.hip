@@ -87,8 +87,10 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gate_up<2, true, true, false>);
         allow_lds(k_mxfp4_gate_up<4, true, true, false>);
         allow_lds(k_mxfp4_gate_up<8, true, true, false>);
-        allow_lds(k_mxfp4_decode_fused<8>);
-        allow_lds(k_mxfp4_decode_fused<0>);
+        allow_lds(k_mxfp4_decode_fused<8, false>);
+        allow_lds(k_mxfp4_decode_fused<0, false>);
+        allow_lds(k_mxfp4_decode_fused<8, true>);
+        allow_lds(k_mxfp4_decode_fused<0, true>);
         allow_lds(k_mxfp4_gemm<true, kGemmMT>);
         allow_lds(k_mxfp4_gemm<false, kGemmMT>);
         allow_lds(k_mxfp4_gemm<true, kGemmMTNarrow>);

@@ -106,45 +106,105 @@ __device__ __forceinline__ float df_load_f32(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// ---- gate/up item ------------------------------------------------------------------------
-__device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint32_t item,
-                                                uint8_t *tiles, float *s_yd,
-                                                float (*s_red)[2][4][64]) {
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t per_token = p.n_slots * p.gu_tiles;
-    const uint32_t t = item / per_token, rem = item - t * per_token;
-    const uint32_t order = rem / p.gu_tiles, j = rem - order * p.gu_tiles;
-    const uint32_t slot = df_slot_of(order, p.n_used, p.n_slots);
-    const uint32_t row0 = df_xcd_contiguous(j, p.gu_tiles) * 16u;
-    df_stamp(p, item, 0);
+// ---- which tokens an item serves ---------------------------------------------------------------
+// With sharing on, the tokens that name one expert in a step (the shared expert: all tokens) are
+// paired in token order, and the items of the first token of a pair also serve the second one,
+// as a second column of the same products; the second token's own items for that expert have
+// nothing to compute.  An expert named by 2 n tokens is then streamed n times instead of 2 n.
+// (crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:621-782 and mxfp4_matvec.hip:568-692
+// group the picks of a few tokens by distinct expert in the same spirit.)
+struct DfCols {          // the two columns of a pair, in LDS for the staging code
+    uint32_t tok[2];
+    uint32_t ms[2];      // token * n_slots + slot of each column
+    float ew[2];
+};
+struct DfPair {
+    uint32_t cnt;        // 0: second token of a pair (nothing to do), 1: alone, 2: with the token below
+    uint32_t t1, ms1;    // the second column
+    float ew0, ew1;      // routing weights of the two columns
+};
 
-    // the token's staged row goes out first: it needs nothing but the token index, and (loads
-    // of a wave return in order) it must not queue behind the weights
-    const uint8_t *xrow = p.xq + (uint64_t)t * p.xq_row_bytes;
-    const uint32_t nq = p.n_sb * 32u;   // 16-byte pieces of the row's tiles
-    constexpr uint32_t kStep = kDfWaves * 64u;
-    uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {};
-    if (tid < nq) ex0 = *(const uint4 *)(xrow + (size_t)tid * 16u);
-    if (tid + kStep < nq) ex1 = *(const uint4 *)(xrow + (size_t)(tid + kStep) * 16u);
-    if (tid + 2u * kStep < nq) ex2 = *(const uint4 *)(xrow + (size_t)(tid + 2u * kStep) * 16u);
-    if (tid + 3u * kStep < nq) ex3 = *(const uint4 *)(xrow + (size_t)(tid + 3u * kStep) * 16u);
-    float early_yd = 0.0f;
-    if (tid < p.n_sb) early_yd = *((const float *)(xrow + (size_t)p.n_sb * 512u) + tid);
-
-    const uint8_t *gate_e, *up_e;
-    float clamp = p.clamp, ew = 1.0f;
-    if (slot < p.n_used) {
-        const int e = p.selected[t * p.n_used + slot];
-        if (e < 0 || (uint32_t)e >= p.n_expert) return;  // empty slot: its down items skip it too
-        gate_e = p.gate + (uint64_t)e * p.gbpe;
-        up_e = p.up + (uint64_t)e * p.ubpe;
-        ew = p.ew[t * p.n_used + slot];
-    } else {
-        gate_e = p.sh_gate;
-        up_e = p.sh_up;
-        clamp = p.sh_clamp;
+// Every wave works the pairing out for itself, in scalar registers: one vector load covers 64
+// (token, slot) picks, a ballot marks those that name expert e, and the tokens before and after
+// t that do so follow from the bit positions -- no LDS, no barrier, and the load goes out next
+// to the one that fetches e, so an item starts its weights no later than without sharing.
+// `e` < 0 names the shared expert (every token has it: tokens 2 i and 2 i + 1 pair up).
+template <bool SHARE>
+__device__ __forceinline__ DfPair df_pair(const DecodeFusedParams &p, uint32_t t, uint32_t slot, int e) {
+    DfPair r{1u, t, t * p.n_slots + slot, 1.0f, 1.0f};
+    if (e < 0) {
+        if (SHARE) {
+            if (t & 1u) {
+                r.cnt = 0u;
+            } else if (t + 1u < p.n_tokens) {
+                r.cnt = 2u;
+                r.t1 = t + 1u;
+                r.ms1 = (t + 1u) * p.n_slots + slot;
+            }
+        }
+        return r;
     }
+    r.ew0 = p.ew[t * p.n_used + slot];
+    if (!SHARE) return r;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t n = p.n_tokens * p.n_used, mine = t * p.n_used, after = mine + p.n_used;
+    uint32_t before = 0u;
+    int next = -1;
+    for (uint32_t base = 0; base < n; base += 64u) {
+        const uint32_t i = base + lane;
+        const int v = i < n ? p.selected[i] : -1;
+        const uint64_t m = __builtin_amdgcn_ballot_w64(v == e);
+        auto below = [&](uint32_t x) -> uint64_t {   // the chunk's entries with index < x
+            return x <= base ? 0ull : x >= base + 64u ? ~0ull : (1ull << (x - base)) - 1ull;
+        };
+        before += (uint32_t)__builtin_popcountll(m & below(mine));
+        const uint64_t later = m & ~below(after);
+        if (next < 0 && later) next = (int)(base + (uint32_t)__builtin_ctzll(later));
+    }
+    if (before & 1u) {
+        r.cnt = 0u;
+    } else if (next >= 0) {
+        r.cnt = 2u;
+        r.t1 = (uint32_t)next / p.n_used;
+        r.ms1 = r.t1 * p.n_slots + ((uint32_t)next - r.t1 * p.n_used);
+        r.ew1 = p.ew[next];
+    }
+    return r;
+}
 
+// How an item names its columns: one column held in registers (no sharing: the item's own
+// token), or a stretch of the list in LDS.
+struct DfOneCol {
+    uint32_t t, m;
+    float w;
+    __device__ __forceinline__ uint32_t tok(uint32_t) const { return t; }
+    __device__ __forceinline__ uint32_t ms(uint32_t) const { return m; }
+    __device__ __forceinline__ float ew(uint32_t) const { return w; }
+    __device__ __forceinline__ const uint32_t *tok_list() const { return nullptr; }
+};
+struct DfListCols {
+    const DfCols *c;
+    uint32_t col0;
+    __device__ __forceinline__ uint32_t tok(uint32_t j) const { return c->tok[col0 + j]; }
+    __device__ __forceinline__ uint32_t ms(uint32_t j) const { return c->ms[col0 + j]; }
+    __device__ __forceinline__ float ew(uint32_t j) const { return c->ew[col0 + j]; }
+    __device__ __forceinline__ const uint32_t *tok_list() const { return c->tok + col0; }
+};
+
+// ---- gate/up item ------------------------------------------------------------------------
+// The products of one 16-row tile of gate and of up with NT token columns (col0 .. col0 + n - 1
+// of the item's list), SwiGLU, write-through store of the mid values, the slots' counters.
+// PRE: the single column's staged row was requested by the caller before the weights (ex0..3,
+// early_yd) -- loads of a wave return in order, so the row must not queue behind them.
+template <int NT, bool PRE, typename Cols>
+__device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, const Cols c,
+                                                uint32_t n, const uint8_t *gate_e,
+                                                const uint8_t *up_e, float clamp, uint32_t row0,
+                                                uint8_t *tiles, float *s_yd, float (*s_red)[2][4][64],
+                                                uint4 ex0, uint4 ex1, uint4 ex2, uint4 ex3,
+                                                float early_yd, uint32_t trace_id) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    constexpr uint32_t kStep = kDfWaves * 64u;
     const uint32_t r = lane & 15u, kb = lane >> 4;
     const uint64_t row_stride = (uint64_t)p.n_sb * kSuperBytes;
     const uint8_t *grow = gate_e + (uint64_t)(row0 + r) * row_stride;
@@ -160,23 +220,31 @@ __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint
         u1 = load_wsuper(urow + (uint64_t)b1 * kSuperBytes, kb);
     }
 
-    // rows longer than four pieces per thread take further passes
-    if (tid < nq) *(uint4 *)(tiles + (size_t)tid * 16u) = ex0;
-    if (tid + kStep < nq) *(uint4 *)(tiles + (size_t)(tid + kStep) * 16u) = ex1;
-    if (tid + 2u * kStep < nq) *(uint4 *)(tiles + (size_t)(tid + 2u * kStep) * 16u) = ex2;
-    if (tid + 3u * kStep < nq) *(uint4 *)(tiles + (size_t)(tid + 3u * kStep) * 16u) = ex3;
-    for (uint32_t q = tid + 4u * kStep; q < nq; q += kStep)
-        *(uint4 *)(tiles + (size_t)q * 16u) = *(const uint4 *)(xrow + (size_t)q * 16u);
-    if (tid < p.n_sb) s_yd[tid] = early_yd;
-    for (uint32_t b = tid + kStep; b < p.n_sb; b += kStep)
-        s_yd[b] = *((const float *)(xrow + (size_t)p.n_sb * 512u) + b);
+    if (PRE) {
+        const uint8_t *xrow = p.xq + (uint64_t)c.tok(0) * p.xq_row_bytes;
+        const uint32_t nq = p.n_sb * 32u;   // 16-byte pieces of the row's tiles
+        if (tid < nq) *(uint4 *)(tiles + (size_t)tid * 16u) = ex0;
+        if (tid + kStep < nq) *(uint4 *)(tiles + (size_t)(tid + kStep) * 16u) = ex1;
+        if (tid + 2u * kStep < nq) *(uint4 *)(tiles + (size_t)(tid + 2u * kStep) * 16u) = ex2;
+        if (tid + 3u * kStep < nq) *(uint4 *)(tiles + (size_t)(tid + 3u * kStep) * 16u) = ex3;
+        // rows longer than four pieces per thread take further passes
+        for (uint32_t q = tid + 4u * kStep; q < nq; q += kStep)
+            *(uint4 *)(tiles + (size_t)q * 16u) = *(const uint4 *)(xrow + (size_t)q * 16u);
+        if (tid < p.n_sb) s_yd[tid] = early_yd;
+        for (uint32_t b = tid + kStep; b < p.n_sb; b += kStep)
+            s_yd[b] = *((const float *)(xrow + (size_t)p.n_sb * 512u) + b);
+    } else {
+        stage_copy<NT, kDfWaves * 64>(tiles, s_yd, n, p.n_sb, tid,
+                                      StageMembers{p.xq, p.xq_row_bytes, c.tok_list()});
+    }
     __syncthreads();
-    df_stamp(p, item, 1);
+    df_stamp(p, trace_id, 1);
 
+    const uint32_t col = (lane & 15u) < n ? (lane & 15u) : 0u;
     v4f acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
     auto compute = [&](uint32_t s, const WSuper &g, const WSuper &u) {
-        const BSuper bs = load_bsuper<1>(tiles + (size_t)s * 512u, kb, 0u);
-        const float yd = s_yd[s];
+        const BSuper bs = load_bsuper<NT>(tiles + (size_t)s * 512u * NT, kb, col);
+        const float yd = s_yd[s * NT + col];
         mfma_super(acc_g, g, bs, yd, kb);
         mfma_super(acc_u, u, bs, yd, kb);
     };
@@ -224,19 +292,74 @@ __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint
     s_red[wave][1][2][lane] = acc_u.z;
     s_red[wave][1][3][lane] = acc_u.w;
     __syncthreads();
-    if (tid < 16u) {
-        const uint32_t l = (tid >> 2) * 16u, i = tid & 3u;  // C layout: row 4*(l/16)+i, column l%16
+    if (tid < 16u * n) {
+        const uint32_t rr = tid & 15u, j = tid >> 4;
+        const uint32_t l = (rr >> 2) * 16u + j, i = rr & 3u;  // C layout: row 4*(l/16)+i, column l%16
         float gs = 0.0f, us = 0.0f;
 #pragma unroll
         for (int w = 0; w < kDfWaves; w++) {
             gs += s_red[w][0][i][l];
             us += s_red[w][1][i][l];
         }
-        const uint32_t ms = t * p.n_slots + slot;
-        df_store_f32(p.mid + (uint64_t)ms * p.inter + row0 + tid, swiglu_clamp(gs, us, clamp, ew));
+        const uint32_t ms = c.ms(j);
+        df_store_f32(p.mid + (uint64_t)ms * p.inter + row0 + rr, swiglu_clamp(gs, us, clamp, c.ew(j)));
         // the hint; not ordered behind the stores on purpose (nobody waits here)
-        if (tid == 0)
+        if (rr == 0)
             __hip_atomic_fetch_add(p.slot_done + ms, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <bool SHARE>
+__device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint32_t item,
+                                                uint8_t *tiles, float *s_yd,
+                                                float (*s_red)[2][4][64], DfCols *cols) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t per_token = p.n_slots * p.gu_tiles;
+    const uint32_t t = item / per_token, rem = item - t * per_token;
+    const uint32_t order = rem / p.gu_tiles, j = rem - order * p.gu_tiles;
+    const uint32_t slot = df_slot_of(order, p.n_used, p.n_slots);
+    const uint32_t row0 = df_xcd_contiguous(j, p.gu_tiles) * 16u;
+    df_stamp(p, item, 0);
+
+    // the token's staged row goes out first (see df_gate_up_core)
+    const uint8_t *xrow = p.xq + (uint64_t)t * p.xq_row_bytes;
+    const uint32_t nq = p.n_sb * 32u;
+    constexpr uint32_t kStep = kDfWaves * 64u;
+    uint4 ex0 = {}, ex1 = {}, ex2 = {}, ex3 = {};
+    if (tid < nq) ex0 = *(const uint4 *)(xrow + (size_t)tid * 16u);
+    if (tid + kStep < nq) ex1 = *(const uint4 *)(xrow + (size_t)(tid + kStep) * 16u);
+    if (tid + 2u * kStep < nq) ex2 = *(const uint4 *)(xrow + (size_t)(tid + 2u * kStep) * 16u);
+    if (tid + 3u * kStep < nq) ex3 = *(const uint4 *)(xrow + (size_t)(tid + 3u * kStep) * 16u);
+    float early_yd = 0.0f;
+    if (tid < p.n_sb) early_yd = *((const float *)(xrow + (size_t)p.n_sb * 512u) + tid);
+
+    const uint8_t *gate_e, *up_e;
+    float clamp = p.clamp;
+    int e = -1;
+    if (slot < p.n_used) {
+        e = p.selected[t * p.n_used + slot];
+        if (e < 0 || (uint32_t)e >= p.n_expert) return;  // empty slot: its down items skip it too
+        gate_e = p.gate + (uint64_t)e * p.gbpe;
+        up_e = p.up + (uint64_t)e * p.ubpe;
+    } else {
+        gate_e = p.sh_gate;
+        up_e = p.sh_up;
+        clamp = p.sh_clamp;
+    }
+    const DfPair pr = df_pair<SHARE>(p, t, slot, e);
+    if (pr.cnt == 0u) return;   // the token above serves this one
+    if (pr.cnt == 1u) {
+        df_gate_up_core<1, true>(p, DfOneCol{t, t * p.n_slots + slot, pr.ew0}, 1u, gate_e, up_e, clamp, row0,
+                                 tiles, s_yd, s_red, ex0, ex1, ex2, ex3, early_yd, item);
+    } else if (SHARE) {
+        // the pair's two columns in one pass over the tile's weights
+        if (tid == 0) {
+            cols->tok[0] = t; cols->ms[0] = t * p.n_slots + slot; cols->ew[0] = pr.ew0;
+            cols->tok[1] = pr.t1; cols->ms[1] = pr.ms1; cols->ew[1] = pr.ew1;
+        }
+        __syncthreads();
+        df_gate_up_core<2, false>(p, DfListCols{cols, 0u}, 2u, gate_e, up_e, clamp, row0, tiles, s_yd,
+                                  s_red, ex0, ex1, ex2, ex3, early_yd, item);
     }
     df_stamp(p, item, 3);
 }
@@ -284,9 +407,48 @@ __device__ __forceinline__ void df_relay_item(const DecodeFusedParams &p) {
 }
 
 // ---- down item ---------------------------------------------------------------------------
+// Adds up the partial rows of token t for the wave's 16 rows [row0, row0 + 16): picks in slot
+// order, then the shared expert, then a shared expert computed elsewhere and the residual.  The
+// caller is the item of the token's last slot in grid order, so the rows it reads come from
+// items that are running or done.  `own` (lane r < 16: row r) stands in for slot `own_slot`;
+// own_slot >= n_slots reads every slot from memory.
+__device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t t, uint32_t row0,
+                                           float own, uint32_t own_slot) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const float *col = p.partials + (uint64_t)t * p.n_slots * p.hidden + row0 + (lane & 15u);
+    float v[DSX_MAX_SLOTS];
+    for (uint32_t spin = 0;; spin++) {
+        bool missing = false;
+#pragma unroll
+        for (int q = 0; q < DSX_MAX_SLOTS; q++) {
+            v[q] = 0.0f;
+            if ((uint32_t)q < p.n_slots && (uint32_t)q != own_slot && lane < 16u)
+                v[q] = df_load_f32(col + (uint64_t)q * p.hidden);
+        }
+#pragma unroll
+        for (int q = 0; q < DSX_MAX_SLOTS; q++) missing |= __float_as_uint(v[q]) == kMidUnwritten;
+        if (__builtin_amdgcn_ballot_w64(missing) == 0ull) break;   // wave-uniform
+        if (spin > p.spin_limit) {
+            if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusPartialWaitExpired);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+    }
+    if (lane < 16u) {
+        float s = 0.0f;
+#pragma unroll
+        for (int q = 0; q < DSX_MAX_SLOTS; q++)
+            if ((uint32_t)q < p.n_slots) s += (uint32_t)q == own_slot ? own : v[q];
+        const uint64_t o = (uint64_t)t * p.hidden + row0 + lane;
+        if (p.shared_rows) s += p.shared_rows[o];
+        if (p.residual) s += p.residual[o];
+        p.out[o] = s;
+    }
+}
+
 // NSB > 0: inter / 256 == NSB, straight-line code with all NSB super-blocks of the wave's rows in
 // registers; NSB == 0: any inter, in passes of up to 8 super-blocks.
-template <int NSB>
+template <int NSB, bool SHARE>
 __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_t item,
                                              uint8_t *tiles, float *s_yd) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -297,44 +459,66 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
     const uint32_t order = rem / p.dn_blocks, j = rem - order * p.dn_blocks;
     const uint32_t slot = df_slot_of(order, p.n_used, p.n_slots);
     const uint32_t row0 = df_xcd_contiguous(j, p.dn_blocks) * kDfDownRows + wave * 16u;
-    const uint32_t ms = t * p.n_slots + slot;
     const uint32_t r = lane & 15u, kb = lane >> 4;
     const uint32_t trace_id = p.n_gu_items + 1u + item;
+    const bool last = order + 1u == p.n_slots;   // this item adds up the token's rows
     df_stamp(p, trace_id, 0);
 
     const uint8_t *down_e = p.sh_down;
-    bool live = true;
+    int e = -1;
     if (slot < p.n_used) {
-        const int e = p.selected[t * p.n_used + slot];
-        live = e >= 0 && (uint32_t)e < p.n_expert;
-        down_e = p.down + (uint64_t)(live ? e : 0) * p.dbpe;
+        e = p.selected[t * p.n_used + slot];
+        if (e < 0 || (uint32_t)e >= p.n_expert) {
+            // empty slot: contributes zeros (the sum must still wait for the others)
+            if (last) df_combine(p, t, row0, 0.0f, slot);
+            else if (lane < 16u) df_store_f32(p.partials + ((uint64_t)t * p.n_slots + slot) * p.hidden + row0 + lane, 0.0f);
+            df_stamp(p, trace_id, 3);
+            return;
+        }
+        down_e = p.down + (uint64_t)e * p.dbpe;
     }
-    v4f acc = {0.f, 0.f, 0.f, 0.f};
-    if (live) {   // uniform over the workgroup
-        // The wave's share of the slot's mid row (blocks wave, wave + 4, ...) is requested first,
-        // through the caches: when the slot's gate/up tiles finished before this item started --
-        // the usual case, they come earlier in the grid -- the row is complete and nothing below
-        // waits for another workgroup.  (Blocks past the row's end repeat its last block, so
-        // that no load sits behind a condition.)
-        const float *mrow = p.mid + (uint64_t)ms * p.inter;
-        const uint32_t blk0 = min(wave, nsb - 1u), blk1 = min(wave + kDfWaves, nsb - 1u);
-        float4 mv0 = *(const float4 *)(mrow + (size_t)blk0 * 256u + lane * 4u);
-        float4 mv1 = *(const float4 *)(mrow + (size_t)blk1 * 256u + lane * 4u);
+    // column 0's share of the mid row (blocks wave, wave + 4, ...) is requested first, through
+    // the caches: when the slot's gate/up tiles finished before this item started -- the usual
+    // case, they come earlier in the grid -- the row is complete and nothing below waits for
+    // another workgroup.  (Blocks past the row's end repeat its last block, so that no load
+    // sits behind a condition.)  A token served by an earlier one loads the same addresses and
+    // drops them.
+    const uint32_t blk0 = min(wave, nsb - 1u), blk1 = min(wave + kDfWaves, nsb - 1u);
+    const float *mrow0 = p.mid + ((uint64_t)t * p.n_slots + slot) * p.inter;
+    float4 mv0 = *(const float4 *)(mrow0 + (size_t)blk0 * 256u + lane * 4u);
+    float4 mv1 = *(const float4 *)(mrow0 + (size_t)blk1 * 256u + lane * 4u);
 
-        const uint8_t *wrow = down_e + (uint64_t)(row0 + r) * nsb * kSuperBytes;
-        constexpr int kHold = NSB > 0 ? NSB : 8;
-        WSuper w[kHold];
-        // the first part of what this wave will read goes out now, the rest once the mid row is
-        // known to be there
-        const int early = (int)p.dn_early;
+    const uint8_t *wrow = down_e + (uint64_t)(row0 + r) * nsb * kSuperBytes;
+    constexpr int kHold = NSB > 0 ? NSB : 8;
+    WSuper w[kHold];
+    // the first part of what this wave will read goes out now, the rest once the mid row is
+    // known to be there
+    const int early = (int)p.dn_early;
 #pragma unroll
-        for (int b = 0; b < kHold; b++)
-            if ((NSB > 0 || (uint32_t)b < nsb) && b < early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
+    for (int b = 0; b < kHold; b++)
+        if ((NSB > 0 || (uint32_t)b < nsb) && b < early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
 
-        auto landed = [](const float4 &v) {
-            return __float_as_uint(v.x) != kMidUnwritten && __float_as_uint(v.y) != kMidUnwritten &&
-                   __float_as_uint(v.z) != kMidUnwritten && __float_as_uint(v.w) != kMidUnwritten;
-        };
+    const DfPair pr = df_pair<SHARE>(p, t, slot, e);
+    const uint32_t cnt = pr.cnt;
+    if (cnt == 0u) {
+        // the token above computes this one's rows; what is left here is the sum
+        if (last) df_combine(p, t, row0, 0.0f, p.n_slots);
+        df_stamp(p, trace_id, 3);
+        return;
+    }
+
+    auto landed = [](const float4 &v) {
+        return __float_as_uint(v.x) != kMidUnwritten && __float_as_uint(v.y) != kMidUnwritten &&
+               __float_as_uint(v.z) != kMidUnwritten && __float_as_uint(v.w) != kMidUnwritten;
+    };
+    // One column's mid row into LDS tiles [c * nsb, (c + 1) * nsb): wait until it is complete,
+    // quantize it.  v0 / v1: the wave's first two blocks if already requested (column 0).
+    auto stage_column = [&](const uint32_t c, const uint32_t ms, float4 v0, float4 v1, const bool have) {
+        const float *mrow = p.mid + (uint64_t)ms * p.inter;
+        if (!have) {
+            v0 = *(const float4 *)(mrow + (size_t)blk0 * 256u + lane * 4u);
+            v1 = *(const float4 *)(mrow + (size_t)blk1 * 256u + lane * 4u);
+        }
         auto reload = [&](uint32_t blk) {   // bypassing the caches
             const float *src = mrow + (size_t)blk * 256u + lane * 4u;
             float4 v;
@@ -368,109 +552,110 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
                 v = reload(blk);
             }
         };
-        wait_block(mv0, blk0);
-        wait_block(mv1, blk1);
+        wait_block(v0, blk0);
+        wait_block(v1, blk1);
+        if (c == 0u) {
+            // the mid row is there: the rest of the weights goes out
 #pragma unroll
-        for (int b = 0; b < kHold; b++)
-            if ((NSB > 0 || (uint32_t)b < nsb) && b >= early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
-        df_stamp(p, trace_id, 1);
-        if (wave < nsb) quantize_block_to_staged(mv0, lane, tiles + (size_t)blk0 * 512u, s_yd + blk0);
-        if (wave + kDfWaves < nsb) quantize_block_to_staged(mv1, lane, tiles + (size_t)blk1 * 512u, s_yd + blk1);
+            for (int b = 0; b < kHold; b++)
+                if ((NSB > 0 || (uint32_t)b < nsb) && b >= early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
+            df_stamp(p, trace_id, 1);
+        }
+        uint8_t *tl = tiles + (size_t)c * nsb * 512u;
+        float *yd = s_yd + c * nsb;
+        if (wave < nsb) quantize_block_to_staged(v0, lane, tl + (size_t)blk0 * 512u, yd + blk0);
+        if (wave + kDfWaves < nsb) quantize_block_to_staged(v1, lane, tl + (size_t)blk1 * 512u, yd + blk1);
         for (uint32_t blk = wave + 2u * kDfWaves; blk < nsb; blk += kDfWaves) {   // rows of more than 8 blocks
             float4 v = *(const float4 *)(mrow + (size_t)blk * 256u + lane * 4u);
             wait_block(v, blk);
-            quantize_block_to_staged(v, lane, tiles + (size_t)blk * 512u, s_yd + blk);
+            quantize_block_to_staged(v, lane, tl + (size_t)blk * 512u, yd + blk);
         }
-        __syncthreads();
-        df_stamp(p, trace_id, 2);
+    };
+    const uint32_t ms0 = t * p.n_slots + slot, ms1 = pr.ms1;
+    stage_column(0u, ms0, mv0, mv1, true);
+    if (SHARE && cnt > 1u) stage_column(1u, ms1, mv0, mv1, false);   // uniform over the workgroup
+    __syncthreads();
+    df_stamp(p, trace_id, 2);
 
+    // both columns against the weights in one pass (each super-block's registers die as it is used)
+    v4f acc = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t *tl1 = tiles + (size_t)nsb * 512u;
 #pragma unroll
-        for (int b = 0; b < kHold; b++) {
-            if (NSB > 0 || (uint32_t)b < nsb) {
-                const BSuper bs = load_bsuper<1>(tiles + (size_t)b * 512u, kb, 0u);
-                mfma_super(acc, w[b], bs, s_yd[b], kb);
+    for (int b = 0; b < kHold; b++) {
+        if (NSB > 0 || (uint32_t)b < nsb) {
+            const BSuper bs = load_bsuper<1>(tiles + (size_t)b * 512u, kb, 0u);
+            mfma_super(acc, w[b], bs, s_yd[b], kb);
+            if (SHARE && cnt > 1u) {
+                const BSuper bt = load_bsuper<1>(tl1 + (size_t)b * 512u, kb, 0u);
+                mfma_super(acc1, w[b], bt, s_yd[nsb + b], kb);
             }
+            // (keeps the next super-block's LDS reads behind these products: hoisted to the top,
+            // the operands of all super-blocks would be live at once)
+            if (SHARE) asm volatile("" : "+v"(acc), "+v"(acc1) :: "memory");
         }
-        if (NSB == 0) {   // rows longer than 8 super-blocks: the rest in further passes
-            for (uint32_t b0 = 8u; b0 < nsb; b0 += 8u) {
+    }
+    if (NSB == 0) {   // rows longer than 8 super-blocks: the rest in further passes
+        for (uint32_t b0 = 8u; b0 < nsb; b0 += 8u) {
+            WSuper w2[8];
 #pragma unroll
-                for (int b = 0; b < 8; b++)
-                    if (b0 + b < nsb) w[b] = load_wsuper(wrow + (uint64_t)(b0 + b) * kSuperBytes, kb);
+            for (int b = 0; b < 8; b++)
+                if (b0 + b < nsb) w2[b] = load_wsuper(wrow + (uint64_t)(b0 + b) * kSuperBytes, kb);
 #pragma unroll
-                for (int b = 0; b < 8; b++) {
-                    if (b0 + b < nsb) {
-                        const BSuper bs = load_bsuper<1>(tiles + (size_t)(b0 + b) * 512u, kb, 0u);
-                        mfma_super(acc, w[b], bs, s_yd[b0 + b], kb);
+            for (int b = 0; b < 8; b++) {
+                if (b0 + b < nsb) {
+                    const BSuper bs = load_bsuper<1>(tiles + (size_t)(b0 + b) * 512u, kb, 0u);
+                    mfma_super(acc, w2[b], bs, s_yd[b0 + b], kb);
+                    if (SHARE && cnt > 1u) {
+                        const BSuper bt = load_bsuper<1>(tl1 + (size_t)(b0 + b) * 512u, kb, 0u);
+                        mfma_super(acc1, w2[b], bt, s_yd[nsb + b0 + b], kb);
                     }
                 }
             }
         }
     }
 
-    // The wave's 16 sums sit in column 0 of the fragment (lanes 0, 16, 32, 48, four rows each);
+    // A wave's 16 sums sit in column 0 of the fragment (lanes 0, 16, 32, 48, four rows each);
     // lane r < 16 takes row r.
-    const int src_lane = (int)(16u * ((lane & 15u) >> 2));
-    const float c0 = __shfl(acc.x, src_lane, 64), c1 = __shfl(acc.y, src_lane, 64);
-    const float c2 = __shfl(acc.z, src_lane, 64), c3 = __shfl(acc.w, src_lane, 64);
-    const uint32_t ci = lane & 3u;
-    const float own = ci == 0u ? c0 : ci == 1u ? c1 : ci == 2u ? c2 : c3;
-    if (order + 1u != p.n_slots) {
-        // not the token's last item of these rows: leave the partial row (write-through, no
-        // waiting for anything) and go
-        if (lane < 16u) df_store_f32(p.partials + (uint64_t)ms * p.hidden + row0 + lane, own);
-        df_stamp(p, trace_id, 3);
-        return;
+    auto to_rows = [&](const v4f &a) {
+        const int src_lane = (int)(16u * ((lane & 15u) >> 2));
+        const float c0 = __shfl(a.x, src_lane, 64), c1 = __shfl(a.y, src_lane, 64);
+        const float c2 = __shfl(a.z, src_lane, 64), c3 = __shfl(a.w, src_lane, 64);
+        const uint32_t ci = lane & 3u;
+        return ci == 0u ? c0 : ci == 1u ? c1 : ci == 2u ? c2 : c3;
+    };
+    if (SHARE && cnt > 1u) {
+        // the second token's rows: always a partial row -- its own item of its last slot adds
+        // them up, so that every wait points backwards in the grid
+        const float other = to_rows(acc1);
+        if (lane < 16u) df_store_f32(p.partials + (uint64_t)ms1 * p.hidden + row0 + lane, other);
     }
-    // The item of the last slot in grid order adds the rows up: the other slots' partial rows
-    // (pre-filled with the pattern; their items come earlier in the grid, so they are running or
-    // done) in slot order -- picks first, then the shared expert -- with its own sums taken
-    // from registers, plus the residual.
-    const float *col = p.partials + (uint64_t)t * p.n_slots * p.hidden + row0 + (lane & 15u);
-    float v[DSX_MAX_SLOTS];
-    for (uint32_t spin = 0;; spin++) {
-        bool missing = false;
-#pragma unroll
-        for (int q = 0; q < DSX_MAX_SLOTS; q++) {
-            v[q] = 0.0f;
-            if ((uint32_t)q < p.n_slots && (uint32_t)q != slot && lane < 16u)
-                v[q] = df_load_f32(col + (uint64_t)q * p.hidden);
-        }
-#pragma unroll
-        for (int q = 0; q < DSX_MAX_SLOTS; q++) missing |= __float_as_uint(v[q]) == kMidUnwritten;
-        if (__builtin_amdgcn_ballot_w64(missing) == 0ull) break;   // wave-uniform
-        if (spin > p.spin_limit) {
-            if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusPartialWaitExpired);
-            break;
-        }
-        __builtin_amdgcn_s_sleep(8);
-    }
-    if (lane < 16u) {
-        float s = 0.0f;
-#pragma unroll
-        for (int q = 0; q < DSX_MAX_SLOTS; q++)
-            if ((uint32_t)q < p.n_slots) s += (uint32_t)q == slot ? own : v[q];
-        const uint64_t o = (uint64_t)t * p.hidden + row0 + lane;
-        if (p.shared_rows) s += p.shared_rows[o];
-        if (p.residual) s += p.residual[o];
-        p.out[o] = s;
+    const float own = to_rows(acc);
+    if (!last) {
+        // not the token's last slot: leave the partial row (write-through, no waiting)
+        if (lane < 16u) df_store_f32(p.partials + (uint64_t)ms0 * p.hidden + row0 + lane, own);
+    } else {
+        df_combine(p, t, row0, own, slot);
     }
     df_stamp(p, trace_id, 3);
 }
 
-// LDS (dynamic): max(n_sb, n_sb_in) tiles of 512 bytes | as many floats
-template <int NSB>
-__global__ __launch_bounds__(kDfWaves * 64) void k_mxfp4_decode_fused(const DecodeFusedParams p) {
+// LDS (dynamic): max(n_sb (twice that when tokens share experts), n_sb_in) tiles of 512 bytes | as many floats
+template <int NSB, bool SHARE>
+__global__ __launch_bounds__(kDfWaves * 64, 1) void k_mxfp4_decode_fused(const DecodeFusedParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[kDfWaves][2][4][64];
-    const uint32_t n_max = p.n_sb > p.n_sb_in ? p.n_sb : p.n_sb_in;
+    __shared__ DfCols s_cols;
+    // gate/up stages one or two token columns of n_sb tiles, down one column of n_sb_in tiles
+    const uint32_t n_gu = SHARE ? 2u * p.n_sb : p.n_sb, n_dn = SHARE ? 2u * p.n_sb_in : p.n_sb_in;
+    const uint32_t n_max = n_gu > n_dn ? n_gu : n_dn;
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + (size_t)n_max * 512u);
     if (blockIdx.x < p.n_gu_items)
-        df_gate_up_item(p, blockIdx.x, tiles, s_yd, s_red);
+        df_gate_up_item<SHARE>(p, blockIdx.x, tiles, s_yd, s_red, &s_cols);
     else if (blockIdx.x == p.n_gu_items)
         df_relay_item(p);
     else
-        df_down_item<NSB>(p, blockIdx.x - p.n_gu_items - 1u, tiles, s_yd);
+        df_down_item<NSB, SHARE>(p, blockIdx.x - p.n_gu_items - 1u, tiles, s_yd);
 }
 
 }  // namespace dsx

@@ -105,8 +105,9 @@ class MoeLayer:
                                              decode_max_tokens, gemm_narrow_members))
 
     def set_decode(self, fused: int = 0, spin_limit: int = 0):
-        """fused: 1 = one launch for gate/up + down (default), 2 = one launch per stage;
-        spin_limit: bound of the in-kernel waits (include/dsx_moe.h: dsx_moe_layer_set_decode)."""
+        """fused: 1 = one launch for gate/up + down, pairing tokens that name one expert from 4
+        tokens on (default), 3 = never pairing, 4 = pairing from 2 tokens on, 2 = one launch per
+        stage; spin_limit: bound of the in-kernel waits (include/dsx_moe.h: dsx_moe_layer_set_decode)."""
         check(lib().dsx_moe_layer_set_decode(self._h, fused, spin_limit))
 
     def status(self, builtin_scratch: bool = False) -> int:

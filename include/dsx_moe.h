@@ -287,9 +287,15 @@ int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uin
                              uint32_t decode_max_tokens, uint32_t gemm_narrow_members);
 /* Decode path of an all-MXFP4 layer (up to decode_max_tokens tokens); no counterpart in the
  * reference.  fused: 1 = gate/up, mid quantization, down and the slot-order sum in ONE launch
- * whose workgroups hand results to each other through device memory (the default), 2 = one
- * launch per stage, 0 keeps the current value.  spin_limit (0 keeps): bound, in polling rounds
- * of about half a microsecond, of every wait one workgroup does for another. */
+ * whose workgroups hand results to each other through device memory (the default); from 4
+ * tokens on, the tokens of a step that name one expert are paired and the expert is streamed
+ * once per pair (the reference's drafter groups few picks by distinct expert likewise,
+ * crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:621-782); results are bitwise the same
+ * with and without pairing.  3 = the same launch, never pairing; 4 = the same launch, pairing
+ * from 2 tokens on (for steps whose tokens mostly name the same experts, such as the
+ * verification of consecutive draft tokens); 2 = one launch per stage; 0 keeps the current
+ * value.  spin_limit (0 keeps): bound, in polling rounds of about half a microsecond, of every
+ * wait one workgroup does for another. */
 int dsx_moe_layer_set_decode(dsx_moe_layer *layer, uint32_t fused, uint32_t spin_limit);
 /* Measurement aid with no counterpart in the reference: a device buffer of n_items x 4 uint64
  * that the one-launch decode path fills with clock readings (constant 100 MHz counter) per

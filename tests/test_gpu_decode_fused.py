@@ -24,7 +24,9 @@ def _both_modes(s, T, sel_in=None, w_in=None):
     layer = MoeLayer(dw, max(T, 1))
     dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
     outs = {}
-    for mode in (1, 2):   # 1 = one launch, 2 = one launch per stage
+    # 1 = one launch (pairs tokens that name one expert from 4 tokens on), 2 = one launch per
+    # stage, 3 = one launch, never pairing, 4 = one launch, pairing from 2 tokens on
+    for mode in (1, 2, 3, 4):
         layer.set_decode(fused=mode)
         if sel_in is None:
             out, sel, w = layer.run(dx, dl, want_routing=True)
@@ -32,6 +34,9 @@ def _both_modes(s, T, sel_in=None, w_in=None):
             out, sel, w = layer.run(dx, None, selected_in=sel_in, weights_in=w_in, want_routing=True)
         assert layer.status() == 0
         outs[mode] = (out.cpu().numpy(), sel.cpu().numpy(), w.cpu().numpy())
+    # pairing changes which workgroup computes a (token, slot) column, never a value
+    for mode in (1, 4):
+        assert np.array_equal(outs[mode][0], outs[3][0]), f"mode {mode} differs from mode 3"
     return x, outs
 
 
@@ -74,10 +79,63 @@ def test_empty_and_out_of_range_picks_are_empty_slots():
     x, outs = _both_modes(s, T, torch.from_numpy(sel).cuda(), torch.from_numpy(w).cuda())
     clean = np.where((sel < 0) | (sel >= s.n_expert), -1, sel)
     want = ref.moe_forward(H.host_weights(s, experts=np.unique(clean[clean >= 0])), x, clean, w)
-    for mode in (1, 2):
+    for mode in (1, 2, 3, 4):
         out, sel_out, _ = outs[mode]
         assert np.array_equal(sel_out, clean)
         assert H.max_rel(out, want) < REGRESSION, mode
+
+
+def _picks(kind, T, s, rng):
+    """Pinned picks in which tokens name the same experts."""
+    k, E = s.n_used, s.n_expert
+    base = rng.choice(E, k, replace=False).astype(np.int32)
+    if kind == "identical":          # every token: the same experts in the same slots
+        sel = np.tile(base, (T, 1))
+    elif kind == "permuted":         # the same experts, each token in another slot order
+        sel = np.stack([rng.permutation(base) for _ in range(T)])
+    elif kind == "odd":              # one expert named by every token (T odd: one is left alone),
+        others = np.setdiff1d(np.arange(E), base[:1])       # in a slot that moves from token to token
+        sel = np.stack([rng.choice(others, k, replace=False) for _ in range(T)])
+        for t in range(T):
+            sel[t, t % k] = base[0]
+    elif kind == "holes":            # identical picks with empty and out-of-range slots among them
+        sel = np.tile(base, (T, 1))
+        sel[1, 0] = -1
+        sel[T // 2, k - 1] = E + 7
+        if T > 2:
+            sel[T - 1, :] = -1
+    else:
+        raise ValueError(kind)
+    return np.ascontiguousarray(sel, dtype=np.int32)
+
+
+@pytest.mark.parametrize("kind", ["identical", "permuted", "odd", "holes"])
+@pytest.mark.parametrize("T,k", [(2, 4), (5, 4), (7, 8), (12, 8)])   # 12 x 8 picks: two 64-pick ballots
+def test_tokens_that_name_the_same_experts(kind, T, k):
+    """Tokens of one step that name the same expert are paired and the expert is streamed once
+    per pair.  The result must be bitwise what every token gets on its own (modes 1 and 4
+    against mode 3, inside _both_modes) and agree with the oracle and the per-stage path."""
+    s = H.Shape(1024, 512, 32, k, route_scale=2.5, clamp=10.0, seed=930 + T)
+    rng = np.random.default_rng(1000 + T * 10 + k)
+    sel = _picks(kind, T, s, rng)
+    if kind == "odd":
+        for t in range(T):   # a token names an expert at most once
+            assert len(set(sel[t])) == k
+    w = rng.uniform(0.1, 0.9, (T, k)).astype(np.float32)
+    x, outs = _both_modes(s, T, torch.from_numpy(sel).cuda(), torch.from_numpy(w).cuda())
+    clean = np.where((sel < 0) | (sel >= s.n_expert), -1, sel)
+    want = ref.moe_forward(H.host_weights(s, experts=np.unique(clean[clean >= 0])), x, clean, w)
+    for mode in (1, 2, 3, 4):
+        assert H.max_rel(outs[mode][0], want) < REGRESSION, mode
+    # a token's output does not depend on which tokens share the step with it
+    if kind == "identical" and T > 2:
+        layer = MoeLayer(H.device_weights(s), T)
+        layer.set_decode(fused=4)
+        dx = torch.from_numpy(x).cuda()
+        dsel, dw_ = torch.from_numpy(sel).cuda(), torch.from_numpy(w).cuda()
+        alone = layer.run(dx[1:2].contiguous(), None, selected_in=dsel[1:2].contiguous(),
+                          weights_in=dw_[1:2].contiguous()).cpu().numpy()
+        assert np.array_equal(alone[0], outs[4][0][1])
 
 
 def test_repeated_calls_are_bitwise_equal():
