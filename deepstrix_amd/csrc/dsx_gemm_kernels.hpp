@@ -168,6 +168,8 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             a_slab[r][m] = __builtin_amdgcn_readfirstlane((row0[m] + wave * kRowsPerWave + r * 16u) * row_stride);
     // scales: one instruction per row set, lane -> (row lane / 2 of the wave's 32, dword lane % 2)
     const uint32_t sc_fetch = (lane >> 1) * row_stride + 128u + (lane & 1u) * 4u;
+    // The part of an address that all lanes share (row set, fragment, super-block) goes into the
+    // scalar base of the load; the lane's own offset is the same register for every weight load.
     auto issue_a = [&](uint32_t sb) {
 #pragma unroll
         for (int r = 0; r < kGemmRF; r++)
@@ -175,14 +177,25 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             for (int m = 0; m < 2; m++)
 #pragma unroll
                 for (int i = 0; i < 2; i++)
-                    lds_dma16(a_lds + (uint32_t)((r * 2 + m) * 2048 + i * 1024), wbase[m],
-                              a_slab[r][m] + (uint32_t)i * 8u * row_stride + a_fetch + sb * kSuperBytes);
+                    lds_dma16(a_lds + (uint32_t)((r * 2 + m) * 2048 + i * 1024),
+                              wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kSuperBytes), a_fetch);
 #pragma unroll
         for (int m = 0; m < 2; m++)
-            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m],
-                     a_slab[0][m] + sc_fetch + sb * kSuperBytes);
+            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kSuperBytes), sc_fetch);
     };
     constexpr int kALoads = 4 * kGemmRF + 2;  // per wave and super-block
+    // load L of those: 0..7 the halves of the four fragments, 8 and 9 the scales of the row sets
+    auto issue_a_one = [&](int L, uint32_t sb) {
+        if (L < 4 * kGemmRF) {
+            const int f = L >> 1, i = L & 1, r = f >> 1, m = f & 1;
+            lds_dma16(a_lds + (uint32_t)(f * 2048 + i * 1024),
+                      wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kSuperBytes), a_fetch);
+        } else {
+            const int m = L - 4 * kGemmRF;
+            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kSuperBytes), sc_fetch);
+        }
+    };
+    constexpr int kAFirst = 6;  // of them requested during the first half of a super-block
     // read side: lane (row n16, block g4) of fragment f: chunk g4 (first half), 4 + g4 (second)
     const uint32_t sw = ((n16 & 7u) * 8u + (g4 ^ (n16 & 7u))) * 16u;  // within a 1 KB slab
     const uint32_t a_rd = (n16 >> 3) * 1024u + sw;
@@ -220,11 +233,11 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         for (int ii = 0; ii < 2; ii++)
 #pragma unroll
             for (int q = 0; q < 2; q++)
-                lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)((ii * 2 + q) * 1024), p.act,
-                          b_fetch[ii] + sb * 512u + h * 256u + (uint32_t)q * 128u);
+                lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)((ii * 2 + q) * 1024),
+                          p.act + (sb * 512u + h * 256u + (uint32_t)q * 128u), b_fetch[ii]);
     };
     auto issue_yd = [&](uint32_t sb) {  // waves 0 and 1: 64 columns each
-        if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * 512u, p.act, yd_fetch + sb * 4u);
+        if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * 512u, p.act + sb * 4u, yd_fetch);
     };
 
     issue_b(0, 0);
@@ -254,7 +267,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // its input, where it waits, and with the group count as a run-time condition waits for
     // each operand right after requesting it (layer at T=4096: 4.5 -> 4.0 ms).
 #define DSX_PIN() asm volatile("" ::: "memory")
-    auto compute_half = [&](auto hc, auto njc, const uint32_t sb) {
+    auto compute_half = [&](auto hc, auto njc, const uint32_t sb, const bool more) {
         constexpr int h = decltype(hc)::value;
         constexpr int NJ = decltype(njc)::value;
         const uint8_t *half = tiles + h * kGemmHalfBytes;
@@ -303,6 +316,23 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
                     }
                 }
             if (q == 1) yd_prev = yd;
+            // the next super-block's weights, a load or two behind each piece's products: a
+            // request that has to wait for room in the memory pipeline then holds back nothing
+            // that the matrix pipe does not already have
+            {
+                constexpr int kFrom = h == 0 ? 0 : kAFirst, kCnt = h == 0 ? kAFirst : kALoads - kAFirst;
+                constexpr int kSpan = h == 0 ? NP : (NP + 1) / 2;   // the second half's go out early
+                const int lo = pc * kCnt / kSpan, hi = (pc + 1) * kCnt / kSpan;
+                if (pc < kSpan && more) {
+                    // literal indices: the load's registers are picked at compile time
+                    if (0 < kCnt && lo <= 0 && 0 < hi) issue_a_one(kFrom + 0, sb + 1u);
+                    if (1 < kCnt && lo <= 1 && 1 < hi) issue_a_one(kFrom + 1, sb + 1u);
+                    if (2 < kCnt && lo <= 2 && 2 < hi) issue_a_one(kFrom + 2, sb + 1u);
+                    if (3 < kCnt && lo <= 3 && 3 < hi) issue_a_one(kFrom + 3, sb + 1u);
+                    if (4 < kCnt && lo <= 4 && 4 < hi) issue_a_one(kFrom + 4, sb + 1u);
+                    if (5 < kCnt && lo <= 5 && 5 < hi) issue_a_one(kFrom + 5, sb + 1u);
+                }
+            }
         }
         // fold the last group
 #pragma unroll
@@ -325,17 +355,16 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             // the wave's A region is free again once its reads have returned
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             issue_b(sb, 1);
-            if (more) issue_a(sb + 1u);
-            compute_half(std::integral_constant<int, 0>{}, njc, sb);
+            compute_half(std::integral_constant<int, 0>{}, njc, sb, more);
             // the second half of B has landed (the younger weight loads may still be on their way)
-            if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kALoads) : "memory");
+            if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kAFirst) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
             if (more) {
                 issue_b(sb + 1u, 0);
                 issue_yd(sb + 1u);
             }
-            compute_half(std::integral_constant<int, 1>{}, njc, sb);
+            compute_half(std::integral_constant<int, 1>{}, njc, sb, more);
             // everything this wave fetched for the next super-block has landed before the others
             // may read it
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
