@@ -86,6 +86,50 @@ __device__ __forceinline__ void split_q4(uint32_t q, uint32_t &hi_word, uint32_t
 }
 
 // ---------------------------------------------------------------------------------------
+// The activation format of the grouped GEMMs: two planes of FP6 (E2M3) codes.
+//
+// The matrix instruction takes a 6-bit operand at twice the rate of an 8-bit one (measured, two
+// waves per SIMD: 9.2 against 4.8 PFLOP/s with FP4 weights), and both planes of the int8 split
+// fit 6 bits exactly: q = 16 sh + ul with sh = q >> 4 in [-8, 7] and ul = q & 15 in [0, 15]; an
+// E2M3 code c < 16 stands for c / 8 (measured with one-hot probes: codes 0..15 are 0, 0.125, ..
+// 1.875), so the low plane's code is ul, the high plane's |sh| with the sign in bit 5, and the
+// block scales 2^3 (130) and 2^7 (134) restore ul and 16 sh.  The products and sums stay exact.
+//
+// Operand layout (one-hot probes): lane l holds column l % 16, k = 32 (l / 16) + n for code
+// n = 0..31 at bits 6 n of six registers -- one 32-element weight block in nibble order, like
+// the FP4 operand.  In memory a row keeps, per super-block, 384 bytes:
+//   for each 128-k half h:  [plane][block g][16 B]  (128 B)  then  [plane][block g][8 B]  (64 B)
+// the first 16 and the last 8 bytes of the 24-byte operand of (plane, block 4 h + g); plane 0 =
+// high.  The n_sb block scales d follow the tiles.
+// ---------------------------------------------------------------------------------------
+constexpr uint32_t kStaged6Bytes = 384;
+constexpr int kScaleB6High = 134, kScaleB6Low = 130;
+__host__ __device__ inline uint32_t staged6_row_bytes(uint32_t n_sb) {
+    return (n_sb * (kStaged6Bytes + 4u) + 15u) & ~15u;
+}
+// Four int8 values (one per byte of `q`, any order) -> their codes of the high and of the low
+// plane, one per byte, same order.
+__device__ __forceinline__ void split_q4_fp6(uint32_t q, uint32_t &hi_codes, uint32_t &lo_codes) {
+    lo_codes = q & 0x0F0F0F0Fu;
+    const uint32_t n = (q >> 4) & 0x0F0F0F0Fu;   // sh as a two's complement nibble
+    // n < 8: code n;  n >= 8: sh = n - 16 < 0, code 0x20 | (16 - n)
+    constexpr uint32_t kNeg03 = 0x25262728u, kNeg47 = 0x21222324u;
+    const uint32_t s = n & 0x07070707u;
+    const uint32_t neg = __builtin_amdgcn_perm(kNeg47, kNeg03, s);
+    const uint32_t m = ((n >> 3) & 0x01010101u) * 0xFFu;
+    hi_codes = (neg & m) | (s & ~m);
+}
+// Four code bytes -> 24 bits, byte i at bits 6 i.
+__device__ __forceinline__ uint32_t pack_codes4(uint32_t c) {
+    return (c & 0x3Fu) | ((c >> 2) & 0xFC0u) | ((c >> 4) & 0x3F000u) | ((c >> 6) & 0xFC0000u);
+}
+// Byte offset, inside a super-block's 384 bytes, of dword i (0..5) of the operand of
+// (half h, plane, block g).
+__device__ __forceinline__ uint32_t staged6_off(uint32_t h, uint32_t plane, uint32_t g, uint32_t i) {
+    return h * 192u + (i < 4u ? plane * 64u + g * 16u + i * 4u : 128u + plane * 32u + g * 8u + (i - 4u) * 4u);
+}
+
+// ---------------------------------------------------------------------------------------
 // Staged activation tile in LDS, for one super-block (256 k) and NT token columns.
 //
 // Operand layout of the instruction for one 128-k half (measured with one-hot probes):

@@ -36,9 +36,10 @@ constexpr int kGemmRF = 2;                  // 16-row fragments per wave and row
 constexpr int kGemmMT = 128;                // token columns per workgroup (the wide tile)
 constexpr int kGemmMTNarrow = 16;           // ... of the narrow tile: groups of a few members
 constexpr int kGemmAWaveBytes = 2 * kGemmRF * 2048 + 2 * 256;  // a wave's weights of one super-block
-// LDS of a workgroup with MT columns: two half super-blocks of the columns | two rows of 128
-// block scales (the loads that fill them are 64 lanes wide) | the waves' weight regions
-constexpr int gemm_half_bytes(int mt) { return mt * 256; }
+// LDS of a workgroup with MT columns: two half super-blocks of the columns (each: 128 bytes per
+// column of operand heads, then 64 bytes per column of operand tails) | two rows of 128 block
+// scales (the loads that fill them are 64 lanes wide) | the waves' weight regions
+constexpr int gemm_half_bytes(int mt) { return mt * 192; }
 constexpr int gemm_yd_off(int mt) { return 2 * gemm_half_bytes(mt); }
 constexpr int gemm_a_off(int mt) { return gemm_yd_off(mt) + 2 * 128 * (int)sizeof(float); }
 constexpr size_t gemm_lds_bytes(int mt) { return (size_t)gemm_a_off(mt) + kGemmWaves * kGemmAWaveBytes; }
@@ -199,6 +200,11 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // read side: lane (row n16, block g4) of fragment f: chunk g4 (first half), 4 + g4 (second)
     const uint32_t sw = ((n16 & 7u) * 8u + (g4 ^ (n16 & 7u))) * 16u;  // within a 1 KB slab
     const uint32_t a_rd = (n16 >> 3) * 1024u + sw;
+    // tails: column n16's 64 bytes hold chunk (2 plane + g4 / 2) at position chunk ^ (n16 / 4)
+    uint32_t bt_rd[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++)
+        bt_rd[q] = n16 * 64u + ((((uint32_t)q * 2u + (g4 >> 1)) ^ (n16 >> 2)) * 16u) + (g4 & 1u) * 8u;
     // sc: the lane's two scale bytes (block g4 of the first and of the second half), bytes 0 and 1
     struct GemmAFrag { uint4 a0, a1; uint32_t sc; };
     GemmAFrag a_cur[kGemmRF][2];
@@ -215,26 +221,33 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             }
     };
 
-    // B half h of super-block sb: bytes [256 h, 256 h + 256) of each column's 512; its 128-byte
-    // run q (piece 2 h + q) of the 8 columns 8 g .. 8 g + 7 is slab 2 g + q of the half buffer.
-    const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 4096u);
-    uint32_t b_fetch[2];  // column 16 w + 8 ii + l8, chunk c8 of each 128-byte run
+    // B half h of super-block sb: bytes [192 h, 192 h + 192) of each column's 384.  Its first 128
+    // bytes (the 16-byte heads of the operands of both planes and four blocks) of the 8 columns
+    // 8 g .. 8 g + 7 are slab g of the half buffer's first part, fetched and swizzled like the
+    // weights; the 64 bytes of tails of the wave's 16 columns are 1 KB of the second part: lane ->
+    // (column lane / 4, 16-byte chunk (lane % 4) ^ (column / 4)), so that 16 columns read at one
+    // chunk spread over all banks.
+    constexpr uint32_t kTailOff = (uint32_t)MT * 128u;   // of the tails inside a half buffer
+    const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 2048u);
+    const uint32_t bt_lds = __builtin_amdgcn_readfirstlane(lds0 + kTailOff + wave * 1024u);
+    uint32_t b_fetch[2];  // column 16 w + 8 ii + l8, chunk c8 of the 128 bytes of heads
 #pragma unroll
     for (int ii = 0; ii < 2; ii++)
         b_fetch[ii] = s_src[(wave * 16u + ii * 8u + l8) & (uint32_t)(MT - 1)] * p.act_row_bytes + c8 * 16u;
-    const uint32_t yd_fetch = s_src[tid & (uint32_t)(MT - 1)] * p.act_row_bytes + p.n_sb * 512u;
+    const uint32_t bt_fetch = s_src[(wave * 16u + (lane >> 2)) & (uint32_t)(MT - 1)] * p.act_row_bytes + 128u +
+                              (((lane & 3u) ^ ((lane >> 4) & 3u)) * 16u);
+    const uint32_t yd_fetch = s_src[tid & (uint32_t)(MT - 1)] * p.act_row_bytes + p.n_sb * kStaged6Bytes;
     const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 256u);
     // a wave whose 16 columns lie past the end of a short group fetches nothing (nobody reads
     // them: the column loop stops at the last group that holds a real column)
     const bool b_live = wave * 16u < cnt;
     auto issue_b = [&](uint32_t sb, uint32_t h) {  // into half buffer h
         if (!b_live) return;
+        const uint8_t *src = p.act + (sb * kStaged6Bytes + h * 192u);
 #pragma unroll
         for (int ii = 0; ii < 2; ii++)
-#pragma unroll
-            for (int q = 0; q < 2; q++)
-                lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)((ii * 2 + q) * 1024),
-                          p.act + (sb * 512u + h * 256u + (uint32_t)q * 128u), b_fetch[ii]);
+            lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)(ii * 1024), src, b_fetch[ii]);
+        lds_dma16(bt_lds + h * kGemmHalfBytes, src, bt_fetch);
     };
     auto issue_yd = [&](uint32_t sb) {  // waves 0 and 1: 64 columns each
         if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * 512u, p.act + sb * 4u, yd_fetch);
@@ -272,9 +285,12 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         constexpr int NJ = decltype(njc)::value;
         const uint8_t *half = tiles + h * kGemmHalfBytes;
         const float *yds = s_yd + (sb & 1u) * 128u;
+        // the operand of (column group j, plane q): 16 bytes of head, 8 of tail
         auto load_piece = [&](int j, int q) -> v8i {
-            const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 2u + (uint32_t)q) * 1024u + sw;
-            return b_operand(half, cb, cb ^ 64u);
+            const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 1024u + sw) ^ ((uint32_t)q * 64u);
+            const uint4 hd = *(const uint4 *)(half + cb);
+            const uint2 tl = *(const uint2 *)(half + kTailOff + (uint32_t)j * 1024u + bt_rd[q]);
+            return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
         };
         v4f c[kGemmRF][2];
         // piece p = 2 j + q alternates between two operand registers
@@ -309,10 +325,10 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
                             asm volatile("" : "+v"(a));
                         }
                         c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                            av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 0, h, (int)w.sc, 0, 131);
+                            av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 2, h, (int)w.sc, 0, kScaleB6High);
                     } else {
                         c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                            av, bq, c[r][m], 4, 0, h, (int)w.sc, 0, 127);
+                            av, bq, c[r][m], 4, 2, h, (int)w.sc, 0, kScaleB6Low);
                     }
                 }
             if (q == 1) yd_prev = yd;
@@ -467,21 +483,21 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         }
         s_iscale[tid] = iscale;
         if (tid < cnt)
-            *(float *)(p.midq + (uint64_t)s_dest[tid] * p.out_row_bytes + (uint64_t)n_blk_out * 512u +
+            *(float *)(p.midq + (uint64_t)s_dest[tid] * p.out_row_bytes + (uint64_t)n_blk_out * kStaged6Bytes +
                        rt * 4u) = d;
     }
     __syncthreads();
     // Rows 16r + 4*g4 + q of fragments r = 2*rho, 2*rho + 1 are the nibble positions
-    // 8*g4 .. 8*g4+7 of 32-element block (kGemmRF / 2) * wave + rho: 8 consecutive bytes of each plane of
-    // the staged tile (byte 2*(q & 1) + (r & 1) of dword q / 2).
-    const uint32_t plane_step = tile_off<1>(0, 1, 0, 0, 0);
+    // 8*g4 .. 8*g4+7 of 32-element block (kGemmRF / 2) * wave + rho (position 4 (q / 2) +
+    // 2 (q & 1) + r & 1): 48 bits of each plane's 24-byte operand, at bit 48 g4.  Dwords 0 and 1
+    // of the operand come from the lanes g4 = 0 and 1, dword 2 from g4 = 1, dwords 3 and 4 from
+    // g4 = 2 and 3, dword 5 from g4 = 3: every lane fetches the low word of the lane 16 above.
 #pragma unroll
     for (int j = 0; j < kGemmCG; j++) {
         const uint32_t col = j * 16u + n16;
         const float iscale = s_iscale[col];
 #pragma unroll
         for (int rho = 0; rho < kGemmRF / 2; rho++) {
-            // dword q / 2 of a plane holds bytes 2 * (q & 1) + rr
             uint32_t qw[2] = {0u, 0u};
 #pragma unroll
             for (int rr = 0; rr < 2; rr++) {
@@ -495,16 +511,26 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
                     qw[q >> 1] |= ((uint32_t)qi & 0xFFu) << ((uint32_t)(2 * (q & 1) + rr) * 8u);
                 }
             }
-            uint32_t hw[2], lw[2];
-            split_q4(qw[0], hw[0], lw[0]);
-            split_q4(qw[1], hw[1], lw[1]);
-            if (col >= cnt) continue;
+            uint32_t hc[2], lc[2];
+            split_q4_fp6(qw[0], hc[0], lc[0]);
+            split_q4_fp6(qw[1], hc[1], lc[1]);
             const uint32_t b32 = wave * (kGemmRF / 2) + rho;
-            const uint32_t hh = b32 >> 2, bb = b32 & 3u;
-            const uint32_t toff = tile_off<1>(hh, 0, bb >> 1, 2u * (bb & 1u) + (g4 >> 1), 0) + (g4 & 1u) * 8u;
-            uint8_t *dst = p.midq + (uint64_t)s_dest[col] * p.out_row_bytes + (uint64_t)rt * 512u + toff;
-            *(uint2 *)(dst) = make_uint2(hw[0], hw[1]);
-            *(uint2 *)(dst + plane_step) = make_uint2(lw[0], lw[1]);
+            uint8_t *dst = p.midq + (uint64_t)s_dest[col] * p.out_row_bytes + (uint64_t)rt * kStaged6Bytes;
+#pragma unroll
+            for (int plane = 0; plane < 2; plane++) {
+                const uint32_t g0 = pack_codes4(plane == 0 ? hc[0] : lc[0]);
+                const uint32_t g1 = pack_codes4(plane == 0 ? hc[1] : lc[1]);
+                const uint32_t lo = g0 | (g1 << 24), hi = g1 >> 8;            // the lane's 48 bits
+                const uint32_t up = (uint32_t)__shfl((int)lo, (int)((lane + 16u) & 63u), 64);
+                if (col >= cnt) continue;
+                const uint32_t base = (g4 >> 1) * 3u;   // first operand dword of the lane pair
+                if ((g4 & 1u) == 0u) {
+                    *(uint32_t *)(dst + staged6_off(b32 >> 2, plane, b32 & 3u, base)) = lo;
+                    *(uint32_t *)(dst + staged6_off(b32 >> 2, plane, b32 & 3u, base + 1u)) = hi | (up << 16);
+                } else {
+                    *(uint32_t *)(dst + staged6_off(b32 >> 2, plane, b32 & 3u, base + 2u)) = (lo >> 16) | (hi << 16);
+                }
+            }
         }
     }
 }

@@ -427,6 +427,7 @@ struct FrontParams {
     float scale, eps;
     uint32_t mode, n_group, topk_group;
     uint32_t n_tokens, n_sb, xp_row_bytes, n_fill, fill_value, route;
+    uint32_t fp6;   // staged rows in the grouped GEMMs' format (FP6 planes, 384 bytes per super-block)
 };
 
 __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParams p) {
@@ -454,7 +455,11 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
         if (blk + step < n_blk) nxt = *(const float4 *)(p.x + (uint64_t)(blk + step) * 256u + lane * 4u);
         const uint32_t t = blk / p.n_sb, b = blk - t * p.n_sb;
         uint8_t *row = p.xp + (uint64_t)t * p.xp_row_bytes;
-        quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
+        if (p.fp6)
+            quantize_block_to_staged6(v, lane, row + (size_t)b * kStaged6Bytes,
+                                      (float *)(row + (size_t)p.n_sb * kStaged6Bytes) + b);
+        else
+            quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
         v = nxt;
     }
     if (p.sel_in != nullptr)

@@ -142,4 +142,40 @@ __device__ __forceinline__ void quantize_block_to_staged(float4 v, uint32_t lane
     if (lane == 0) *d_out = r.d;
 }
 
+// The same block in the grouped GEMMs' format (FP6 planes, dsx_device.hpp): `sb` points at the
+// super-block's 384 bytes.  The lane that builds nibble positions 4 d .. 4 d + 3 packs their codes
+// into 24 bits; dword i of a block's 24-byte operand takes the tail of group i and the head of
+// group i + 1 (groups 0..3 make dwords 0..2, groups 4..7 dwords 3..5), so the lanes of groups
+// 0, 1, 2 and 4, 5, 6 each fetch their neighbour's group and store one dword per plane.
+__device__ __forceinline__ void quantize_block_to_staged6(float4 v, uint32_t lane, uint8_t *sb,
+                                                          float *d_out) {
+    const Q8kQuant r = q8k_quantize_lane(v, lane);
+    const uint32_t mine = (uint32_t)(r.q[0] & 0xFF) | ((uint32_t)(r.q[1] & 0xFF) << 8) |
+                          ((uint32_t)(r.q[2] & 0xFF) << 16) | ((uint32_t)(r.q[3] & 0xFF) << 24);
+    const uint32_t other = (uint32_t)__shfl_xor((int)mine, 4, 64);
+    const uint32_t m = lane & 7u;
+    const bool low_half = m < 4u;
+    const uint32_t lo4 = low_half ? mine : other;
+    const uint32_t hi4 = low_half ? other : mine;
+    const uint32_t packed = __builtin_amdgcn_perm(hi4, lo4, low_half ? 0x05010400u : 0x07030602u);
+    uint32_t hc, lc;
+    split_q4_fp6(packed, hc, lc);
+    const uint32_t gh = pack_codes4(hc), gl = pack_codes4(lc);
+    const uint32_t d = 2u * (m & 3u) + (low_half ? 0u : 1u);
+    // the lane that holds group d + 1 of the same block: d + 1 even -> m' = (d + 1) / 2, odd -> d / 2 + 4
+    const uint32_t dn = (d + 1u) & 7u;
+    const uint32_t src = (lane & ~7u) + ((dn & 1u) ? (dn >> 1) + 4u : (dn >> 1));
+    const uint32_t nh = (uint32_t)__shfl((int)gh, (int)src, 64);
+    const uint32_t nl = (uint32_t)__shfl((int)gl, (int)src, 64);
+    const uint32_t i = d & 3u;
+    if (i < 3u) {
+        const uint32_t b32 = lane >> 3, idx = (d >> 2) * 3u + i;
+        const uint32_t wh = (gh >> (8u * i)) | (nh << (24u - 8u * i));
+        const uint32_t wl = (gl >> (8u * i)) | (nl << (24u - 8u * i));
+        *(uint32_t *)(sb + staged6_off(b32 >> 2, 0, b32 & 3u, idx)) = wh;
+        *(uint32_t *)(sb + staged6_off(b32 >> 2, 1, b32 & 3u, idx)) = wl;
+    }
+    if (lane == 0) *d_out = r.d;
+}
+
 }  // namespace dsx
