@@ -124,22 +124,23 @@ def prefill_leg(dw, base, H, torch, np, T=4096, reps=5):
     dt = (time.perf_counter() - t0) / reps
     flops = 2.0 * T * (s.n_used + 1) * 3 * s.hidden * s.inter
     del layer
-    # the bound of this arithmetic: every product is two FP8-rate instructions (the int8
-    # activations as two exact FP8 planes), so the useful rate tops out at half the FP8 peak
+    # the bound of this arithmetic: every product is two instructions at the FP6/FP4 rate (the
+    # int8 activations as two exact planes of FP6 codes), so the useful rate tops out at half the
+    # MXFP4 peak
     roof = {"bound": "mfma", "kernel": "k_mxfp4_gemm<true,128> + k_mxfp4_gemm<false,128> (whole layer, "
-            "wall clock)", "achieved": flops / dt / 1e12, "peak": FP8_MFMA_PEAK / 1e12,
-            "unit": "TFLOP/s", "frac": flops / dt / FP8_MFMA_PEAK,
-            "frac_of_two_plane_bound": 2.0 * flops / dt / FP8_MFMA_PEAK,
-            "frac_of_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK, "traffic": None,
+            "wall clock)", "achieved": flops / dt / 1e12, "peak": MXFP4_MFMA_PEAK / 1e12,
+            "unit": "TFLOP/s", "frac": flops / dt / MXFP4_MFMA_PEAK,
+            "frac_of_two_plane_bound": 2.0 * flops / dt / MXFP4_MFMA_PEAK,
+            "frac_of_fp8_peak": flops / dt / FP8_MFMA_PEAK, "traffic": None,
             "algorithmic_flop_per_launch": flops}
     return {"roofline": roof, "tokens_per_s": T / dt, "ms_per_layer": dt * 1e3, "zipf_alpha": alpha,
             "top10pct_share": frac, "max_group": int(cnt.max()), "empty_experts": int((cnt == 0).sum()),
             "column_tiles_of_128": int(np.ceil(cnt / 128).sum()) + T // 128,
             "useful_flop": flops, "useful_TFLOPs": flops / dt / 1e12,
-            "mfma_issued": "v_mfma_scale_f32_16x16x128_f8f6f4, A = FP4 weights, B = FP8 planes of the "
-                           "int8 activations (two instructions per product)",
+            "mfma_issued": "v_mfma_scale_f32_16x16x128_f8f6f4, A = FP4 weights, B = FP6 (E2M3) planes of "
+                           "the int8 activations (two instructions per product, each at the FP4 rate)",
             "mfma_frac_useful_vs_fp8_peak": flops / dt / FP8_MFMA_PEAK,
-            "mfma_frac_issued_vs_fp8_peak": 2.0 * flops / dt / FP8_MFMA_PEAK,
+            "mfma_frac_issued_vs_mxfp4_peak": 2.0 * flops / dt / MXFP4_MFMA_PEAK,
             "mfma_frac_useful_vs_mxfp4_peak": flops / dt / MXFP4_MFMA_PEAK}
 
 

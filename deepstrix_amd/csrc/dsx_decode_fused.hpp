@@ -67,6 +67,7 @@ struct DecodeFusedParams {
     float *out;                      // [n_tokens, hidden]
     const float *residual;           // [n_tokens, hidden] or null; may alias out
     const float *shared_rows;        // [n_tokens, hidden] or null: a shared expert computed elsewhere
+    uint32_t shared_async;           // ... by another stream, into rows marked unwritten: wait for them
     uint32_t *slot_done;             // [n_tokens, n_slots], zero on entry
     uint32_t *ready;                 // [n_tokens, n_slots, kDfFan] flags kDfFanStride words apart, zero on entry
     uint32_t dn_early;               // super-blocks of a down item's weights requested before its mid row is checked
@@ -417,8 +418,14 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
     const uint32_t lane = threadIdx.x & 63u;
     const float *col = p.partials + (uint64_t)t * p.n_slots * p.hidden + row0 + (lane & 15u);
     float v[DSX_MAX_SLOTS];
+    float vs = 0.0f;   // the shared expert's value when another stream computes it
+    const uint64_t o = (uint64_t)t * p.hidden + row0 + (lane & 15u);
     for (uint32_t spin = 0;; spin++) {
         bool missing = false;
+        if (p.shared_async && lane < 16u) {
+            vs = df_load_f32(p.shared_rows + o);
+            missing = __float_as_uint(vs) == kMidUnwritten;
+        }
 #pragma unroll
         for (int q = 0; q < DSX_MAX_SLOTS; q++) {
             v[q] = 0.0f;
@@ -439,8 +446,7 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
 #pragma unroll
         for (int q = 0; q < DSX_MAX_SLOTS; q++)
             if ((uint32_t)q < p.n_slots) s += (uint32_t)q == own_slot ? own : v[q];
-        const uint64_t o = (uint64_t)t * p.hidden + row0 + lane;
-        if (p.shared_rows) s += p.shared_rows[o];
+        if (p.shared_rows) s += p.shared_async ? vs : p.shared_rows[o];
         if (p.residual) s += p.residual[o];
         p.out[o] = s;
     }

@@ -83,3 +83,40 @@ def v3_layer():
 def test_v3_shape_with_q8_0_shared_expert(T, v3_layer):
     layer, hw = v3_layer
     _check(V3, layer, hw, T, modes=(1, 2) if T <= 14 else (1,))
+
+
+@pytest.mark.parametrize("T", [2, 4, 12])
+def test_side_stream_shared_expert_under_graph_capture(T, v3_layer):
+    """From two tokens on, the one-launch decode path computes the Q8_0 shared expert on a stream
+    of its own, forked from and joined to the caller's: a capture of the caller's stream must
+    record both branches, and every replay must give what the eager call gives -- bitwise, with
+    the program's own work and synchronizations between the replays."""
+    s = V3
+    layer, hw = v3_layer
+    layer.set_decode(fused=1)
+    x, logits, _ = H.host_inputs(s, T)
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    out = torch.empty((T, s.hidden), dtype=torch.float32, device="cuda")
+    layer.run(dx, dl, out=out)
+    assert layer.status() == 0
+    eager = out.clone()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer.run(dx, dl, out=out)          # warm-up on the capturing stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            layer.run(dx, dl, out=out)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        out.fill_(float(rep))               # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        assert layer.status() == 0
+    # and the eager path still agrees afterwards
+    layer.run(dx, dl, out=out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager)
