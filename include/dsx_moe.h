@@ -331,7 +331,7 @@ int dsx_moe_layer_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
  * DSX_NOALLOC_SCRATCH_BYTES array inside the library's code object; each device holds its own
  * copy from the moment the library is loaded until the process ends, and dsx_init() resolves its
  * address.  Calls whose dsx_moe_layer_workspace_bytes(layer, n_tokens) exceeds the array are
- * refused with DSX_ERR_UNSUPPORTED (at the DeepSeek-V3 shape, 7168 x 2048 with 256 experts and top-8: up to 17 tokens).  Every call on a
+ * refused with DSX_ERR_UNSUPPORTED (at the DeepSeek-V3 shape, 7168 x 2048 with 256 experts and top-8: up to 15 tokens).  Every call on a
  * device shares that device's array: calls that overlap in time on one device (two streams, two
  * layers) race; calls ordered on one stream do not.  Results are those of
  * dsx_moe_layer_forward. */
