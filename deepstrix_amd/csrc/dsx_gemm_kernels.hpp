@@ -113,19 +113,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
 
     const uint32_t wi = (uint32_t)p.work_items[item];
     const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
-    const uint32_t cnt = min((uint32_t)MT, (uint32_t)p.group_count[e] - start);
-    const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
     const bool extra = e >= p.n_expert;
-    const float clamp = extra ? p.sh_clamp : p.clamp;
-    if (tid < (uint32_t)MT) {
-        // columns past the end of the group repeat its last member; they are never stored
-        const uint32_t m = (uint32_t)p.members[mbase + min(tid, cnt - 1u)];
-        const uint32_t dest = gemm_dest_row(m, p.n_tokens, p.n_used);
-        s_dest[tid] = dest;
-        s_src[tid] = PAIR ? (m >> 16) : dest;
-        if (PAIR) s_ew[tid] = (m & 0xFFFFu) >= p.n_used ? 1.0f : p.ew[dest];
-    }
-
     const uint32_t row_stride = p.n_sb * kSuperBytes;
     const uint8_t *wbase[2];
     uint32_t row0[2];
@@ -138,20 +126,9 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         row0[0] = rt * 512u;
         row0[1] = rt * 512u + 256u;
     }
-    __syncthreads();  // s_src visible
 
-    // ---- data movement: global memory -> LDS without passing through registers ------------
-    // A load whose consecutive lanes read consecutive addresses costs the L1 a quarter of what
-    // the matrix instruction's own operand layout (lane -> row lane % 16) costs, because the L1
-    // looks up one cache line per cycle and a group of four lanes then shares a line.  So both
-    // operands are fetched in memory order by LDS-direct loads (lane l of an instruction writes
-    // LDS bytes [16 l, 16 l + 16) of the instruction's 1 KB destination) and read back from
-    // LDS in operand order.  The 16-byte chunk a lane fetches is XOR-swizzled with its row so
-    // that the later reads, 16 rows at a fixed chunk, spread over all banks.
-    //
-    // A, per wave and super-block: 4 fragments x (16 rows x 128 B of nibbles) + 64 rows x 8 B
-    // of scales, private to the wave (no barrier).  B: the 128 columns' 256 B of half a
-    // super-block, shared, double buffered; wave w fetches columns 16 w .. 16 w + 15.
+    // The first super-block of weights depends on the expert and the row tile alone: it is requested
+    // here, so that its trip to memory runs beside the look-ups of the group and its members.
     constexpr uint32_t kRowsPerWave = 16u * kGemmRF;
     static_assert(kGemmRF == 2, "one scale instruction covers the 32 rows of a wave's row set");
     constexpr uint32_t kScaleOff = 2u * kGemmRF * 2048u;
@@ -184,6 +161,34 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         for (int m = 0; m < 2; m++)
             lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kSuperBytes), sc_fetch);
     };
+    issue_a(0);
+
+    const uint32_t cnt = min((uint32_t)MT, (uint32_t)p.group_count[e] - start);
+    const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+    const float clamp = extra ? p.sh_clamp : p.clamp;
+    if (tid < (uint32_t)MT) {
+        // columns past the end of the group repeat its last member; they are never stored
+        const uint32_t m = (uint32_t)p.members[mbase + min(tid, cnt - 1u)];
+        const uint32_t dest = gemm_dest_row(m, p.n_tokens, p.n_used);
+        s_dest[tid] = dest;
+        s_src[tid] = PAIR ? (m >> 16) : dest;
+        if (PAIR) s_ew[tid] = (m & 0xFFFFu) >= p.n_used ? 1.0f : p.ew[dest];
+    }
+
+    __syncthreads();  // s_src visible
+
+    // ---- data movement: global memory -> LDS without passing through registers ------------
+    // A load whose consecutive lanes read consecutive addresses costs the L1 a quarter of what
+    // the matrix instruction's own operand layout (lane -> row lane % 16) costs, because the L1
+    // looks up one cache line per cycle and a group of four lanes then shares a line.  So both
+    // operands are fetched in memory order by LDS-direct loads (lane l of an instruction writes
+    // LDS bytes [16 l, 16 l + 16) of the instruction's 1 KB destination) and read back from
+    // LDS in operand order.  The 16-byte chunk a lane fetches is XOR-swizzled with its row so
+    // that the later reads, 16 rows at a fixed chunk, spread over all banks.
+    //
+    // A, per wave and super-block: 4 fragments x (16 rows x 128 B of nibbles) + 64 rows x 8 B
+    // of scales, private to the wave (no barrier).  B: the 128 columns' 192 B of half a
+    // super-block, shared, double buffered; wave w fetches columns 16 w .. 16 w + 15.
     constexpr int kALoads = 4 * kGemmRF + 2;  // per wave and super-block
     // load L of those: 0..7 the halves of the four fragments, 8 and 9 the scales of the row sets
     auto issue_a_one = [&](int L, uint32_t sb) {
@@ -200,11 +205,9 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // read side: lane (row n16, block g4) of fragment f: chunk g4 (first half), 4 + g4 (second)
     const uint32_t sw = ((n16 & 7u) * 8u + (g4 ^ (n16 & 7u))) * 16u;  // within a 1 KB slab
     const uint32_t a_rd = (n16 >> 3) * 1024u + sw;
-    // tails: column n16's 64 bytes hold chunk (2 plane + g4 / 2) at position chunk ^ (n16 / 4)
-    uint32_t bt_rd[2];
-#pragma unroll
-    for (int q = 0; q < 2; q++)
-        bt_rd[q] = n16 * 64u + ((((uint32_t)q * 2u + (g4 >> 1)) ^ (n16 >> 2)) * 16u) + (g4 & 1u) * 8u;
+    // tails: column n16's 64 bytes hold chunk (2 plane + g4 / 2) at position chunk ^ (n16 / 4);
+    // the two planes' positions differ in one address bit
+    const uint32_t bt_rd = n16 * 64u + (((g4 >> 1) ^ (n16 >> 2)) * 16u) + (g4 & 1u) * 8u;
     // sc: the lane's two scale bytes (block g4 of the first and of the second half), bytes 0 and 1
     struct GemmAFrag { uint4 a0, a1; uint32_t sc; };
     GemmAFrag a_cur[kGemmRF][2];
@@ -255,7 +258,6 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
 
     issue_b(0, 0);
     issue_yd(0);
-    issue_a(0);
 
     v4f acc[kGemmRF][2][kGemmCG];
 #pragma unroll
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         auto load_piece = [&](int j, int q) -> v8i {
             const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 1024u + sw) ^ ((uint32_t)q * 64u);
             const uint4 hd = *(const uint4 *)(half + cb);
-            const uint2 tl = *(const uint2 *)(half + kTailOff + (uint32_t)j * 1024u + bt_rd[q]);
+            const uint2 tl = *(const uint2 *)(half + kTailOff + (uint32_t)j * 1024u + (bt_rd ^ ((uint32_t)q * 32u)));
             return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
         };
         v4f c[kGemmRF][2];
