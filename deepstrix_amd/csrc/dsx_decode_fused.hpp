@@ -10,8 +10,9 @@
 // (a wave holds its 16 rows x 8 super-blocks in registers) and only then waits, so while the last
 // gate/up items drain, the slots they free fill with down items whose weights are already on
 // their way: the memory pipe sees one stream of gate, up and down weights with no kernel
-// boundary in it.  The item of a token's last slot adds the slots' partial rows in slot order (crates/v4flash-kernels/kernels/q2_k_accumulate_matvec_par.hip:724-729)
-// plus the residual and writes the output.
+// boundary in it.  The item of a token's last slot adds the slots' partial rows in slot order
+// (crates/v4flash-kernels/kernels/q2_k_accumulate_matvec_par.hip:724-729), then a shared expert's
+// rows computed elsewhere and the residual, and writes the output.
 //
 // Hand-off between workgroups (they may run on different XCDs, whose L2 caches are not coherent
 // with each other):

@@ -6,15 +6,19 @@
 // weight rows with those 128 columns over the whole k range:
 //   gate/up (PAIR):  256 rows of gate and the same 256 rows of up; the epilogue applies the
 //                    clamped SwiGLU and the routing weight, quantizes the 256 results of
-//                    every column as one Q8_K block and writes it in the staged format
+//                    every column as one Q8_K block and writes it as the FP6 row
 //                    that `down` reads -- the f32 `mid` never goes to memory;
 //   down:            512 rows; the epilogue stores f32 partial rows, one per (token, slot).
 // Wave w owns rows [32 w, 32 w + 32) of both row sets and all 128 columns: 2 x 2 x 8 = 32
 // accumulator fragments.  Column groups past the end of a short group are skipped.
 //
+// The activations come as two planes of FP6 (E2M3) codes (dsx_device.hpp): the matrix
+// instruction takes a 6-bit operand in half the cycles of an 8-bit one, and the int8 split
+// q = 16 (q >> 4) + (q & 15) stays exact in it.
+//
 // The kernel is bound by the bytes that pass through the CU's L1, which serves requests in
 // order: one HBM miss holds back the L2 hits behind it, so every byte moves at about HBM
-// speed (about 19 GB/s per CU) whether or not it hits in L2.  Hence the wide tile (weight
+// speed (19-26 GB/s per CU) whether or not it hits in L2.  Hence the wide tile (weight
 // bytes per product halve against 64 columns) and loads in memory order (see below).
 //
 // The Q8_K block scale d of the activations differs per (column, super-block), so the
