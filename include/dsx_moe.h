@@ -278,8 +278,9 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
  * path (128 token columns per work item, shared expert as an extra group; a Q8_0 down matrix
  * takes the int8 grouped GEMM); an all-MXFP4 layer whose GEMMs use the narrow tile (below)
  * switches at 11/16 of it.
- * decode_max_tokens (default 14): up to this many tokens, an all-MXFP4 layer runs the one-token decode
- * kernels once per token inside the same launches (no grouping by expert).
+ * decode_max_tokens (default 16): up to this many tokens, an all-MXFP4 layer runs the decode path
+ * (dsx_moe_layer_set_decode: every token on its own picks, no grouping by expert; the one-launch
+ * form serves at most 16 tokens, beyond that the decode kernels run once per stage).
  * gemm_narrow_members: while the picks per expert average less than this, the all-MXFP4
  * grouped GEMMs use 16 token columns per work item and two workgroups per CU (they only
  * stream weights then); 1 turns the narrow tile off. */
