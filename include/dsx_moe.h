@@ -274,16 +274,15 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
                                      void *down_end);
 /* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens: from this many tokens on, a layer with MXFP4 gate/up runs the grouped-GEMM
- * path (128 token columns per work item, shared expert as an extra group; a Q8_0 down matrix
- * takes the int8 grouped GEMM); an all-MXFP4 layer whose GEMMs use the narrow tile (below)
- * switches at 11/16 of it.
+ * gemm_min_tokens (default 100): from this many tokens on, a layer with MXFP4 gate/up runs the
+ * grouped-GEMM path (128 token columns per work item, shared expert as an extra group; a Q8_0
+ * down matrix takes the int8 grouped GEMM); an all-MXFP4 layer whose GEMMs use the narrow tile
+ * (below) switches at 11/16 of it.
  * decode_max_tokens (default 16): up to this many tokens, an all-MXFP4 layer runs the decode path
  * (dsx_moe_layer_set_decode: every token on its own picks, no grouping by expert; the one-launch
  * form serves at most 16 tokens, beyond that the decode kernels run once per stage).
- * gemm_narrow_members: while the picks per expert average less than this, the all-MXFP4
- * grouped GEMMs use 16 token columns per work item and two workgroups per CU (they only
- * stream weights then); 1 turns the narrow tile off. */
+ * gemm_narrow_members (default 1 = never): while the picks per expert average less than this,
+ * the all-MXFP4 grouped GEMMs use 16 token columns per work item and two workgroups per CU. */
 int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
                              uint32_t decode_max_tokens, uint32_t gemm_narrow_members);
 /* Decode path of an all-MXFP4 layer (up to decode_max_tokens tokens); no counterpart in the
