@@ -98,14 +98,15 @@ __device__ __forceinline__ void split_q4(uint32_t q, uint32_t &hi_word, uint32_t
 // Operand layout (one-hot probes): lane l holds column l % 16, k = 32 (l / 16) + n for code
 // n = 0..31 at bits 6 n of six registers -- one 32-element weight block in nibble order, like
 // the FP4 operand.  In memory a row keeps, per super-block, 384 bytes:
-//   for each 128-k half h:  [plane][block g][16 B]  (128 B)  then  [plane][block g][8 B]  (64 B)
+//   [half h][plane][block g][16 B]  (2 x 128 B)  then  [half h][plane][block g][8 B]  (2 x 64 B)
 // the first 16 and the last 8 bytes of the 24-byte operand of (plane, block 4 h + g); plane 0 =
-// high.  The n_sb block scales d follow the tiles.
+// high.  Rows are 128 bytes apart in multiples, so the 128-byte runs are whole cache lines.  The
+// n_sb block scales d follow the tiles.
 // ---------------------------------------------------------------------------------------
 constexpr uint32_t kStaged6Bytes = 384;
 constexpr int kScaleB6High = 134, kScaleB6Low = 130;
 __host__ __device__ inline uint32_t staged6_row_bytes(uint32_t n_sb) {
-    return (n_sb * (kStaged6Bytes + 4u) + 15u) & ~15u;
+    return (n_sb * (kStaged6Bytes + 4u) + 127u) & ~127u;
 }
 // Four int8 values (one per byte of `q`, any order) -> their codes of the high and of the low
 // plane, one per byte, same order.
@@ -126,7 +127,7 @@ __device__ __forceinline__ uint32_t pack_codes4(uint32_t c) {
 // Byte offset, inside a super-block's 384 bytes, of dword i (0..5) of the operand of
 // (half h, plane, block g).
 __device__ __forceinline__ uint32_t staged6_off(uint32_t h, uint32_t plane, uint32_t g, uint32_t i) {
-    return h * 192u + (i < 4u ? plane * 64u + g * 16u + i * 4u : 128u + plane * 32u + g * 8u + (i - 4u) * 4u);
+    return i < 4u ? h * 128u + plane * 64u + g * 16u + i * 4u : 256u + h * 64u + plane * 32u + g * 8u + (i - 4u) * 4u;
 }
 
 // ---------------------------------------------------------------------------------------

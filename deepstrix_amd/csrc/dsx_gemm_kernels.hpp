@@ -228,12 +228,12 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             }
     };
 
-    // B half h of super-block sb: bytes [192 h, 192 h + 192) of each column's 384.  Its first 128
-    // bytes (the 16-byte heads of the operands of both planes and four blocks) of the 8 columns
-    // 8 g .. 8 g + 7 are slab g of the half buffer's first part, fetched and swizzled like the
-    // weights; the 64 bytes of tails of the wave's 16 columns are 1 KB of the second part: lane ->
-    // (column lane / 4, 16-byte chunk (lane % 4) ^ (column / 4)), so that 16 columns read at one
-    // chunk spread over all banks.
+    // B half h of super-block sb: of each column's 384 bytes the 128 at 128 h (the 16-byte heads of
+    // the operands of both planes and four blocks) and the 64 at 256 + 64 h (their 8-byte tails).
+    // The heads of the 8 columns 8 g .. 8 g + 7 are slab g of the half buffer's first part, fetched
+    // and swizzled like the weights; the tails of the wave's 16 columns are 1 KB of the second
+    // part: lane -> (column lane / 4, 16-byte chunk (lane % 4) ^ (column / 4)), so that 16 columns
+    // read at one chunk spread over all banks.
     constexpr uint32_t kTailOff = (uint32_t)MT * 128u;   // of the tails inside a half buffer
     const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 2048u);
     const uint32_t bt_lds = __builtin_amdgcn_readfirstlane(lds0 + kTailOff + wave * 1024u);
@@ -241,7 +241,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
 #pragma unroll
     for (int ii = 0; ii < 2; ii++)
         b_fetch[ii] = s_src[(wave * 16u + ii * 8u + l8) & (uint32_t)(MT - 1)] * p.act_row_bytes + c8 * 16u;
-    const uint32_t bt_fetch = s_src[(wave * 16u + (lane >> 2)) & (uint32_t)(MT - 1)] * p.act_row_bytes + 128u +
+    const uint32_t bt_fetch = s_src[(wave * 16u + (lane >> 2)) & (uint32_t)(MT - 1)] * p.act_row_bytes + 256u +
                               (((lane & 3u) ^ ((lane >> 4) & 3u)) * 16u);
     const uint32_t yd_fetch = s_src[tid & (uint32_t)(MT - 1)] * p.act_row_bytes + p.n_sb * kStaged6Bytes;
     const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 256u);
@@ -250,11 +250,11 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     const bool b_live = wave * 16u < cnt;
     auto issue_b = [&](uint32_t sb, uint32_t h) {  // into half buffer h
         if (!b_live) return;
-        const uint8_t *src = p.act + (sb * kStaged6Bytes + h * 192u);
+        const uint8_t *src = p.act + (sb * kStaged6Bytes + h * 128u);
 #pragma unroll
         for (int ii = 0; ii < 2; ii++)
             lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)(ii * 1024), src, b_fetch[ii]);
-        lds_dma16(bt_lds + h * kGemmHalfBytes, src, bt_fetch);
+        lds_dma16(bt_lds + h * kGemmHalfBytes, p.act + (sb * kStaged6Bytes + h * 64u), bt_fetch);
     };
     auto issue_yd = [&](uint32_t sb) {  // waves 0 and 1: 64 columns each
         if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * 512u, p.act + sb * 4u, yd_fetch);
