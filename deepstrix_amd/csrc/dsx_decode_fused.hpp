@@ -40,6 +40,7 @@
 
 #include "dsx_device.hpp"
 #include "dsx_expert_kernels.hpp"
+#include "dsx_q8_0_kernels.hpp"
 #include "dsx_quant.hpp"
 
 namespace dsx {
@@ -55,6 +56,11 @@ struct DecodeFusedParams {
     // gate/up
     const uint8_t *gate, *up;        // [n_expert] experts, gbpe / ubpe apart
     const uint8_t *sh_gate, *sh_up;  // shared expert (slot n_used) or null
+    // The shared expert may be kept in Q8_0 (engine rows [blocks x f16 d][blocks x 32 i8]) and be
+    // narrower than the routed ones: sh_q8 != 0, sh_inter <= inter, the tokens also as Q8_0 rows
+    uint32_t sh_q8, sh_inter;
+    const uint8_t *xq8;              // [n_tokens] Q8_0 activation rows, xq8_row_bytes apart
+    uint32_t xq8_row_bytes;
     uint64_t gbpe, ubpe;
     const uint8_t *xq;               // [n_tokens] staged rows, xq_row_bytes apart
     const float *ew;                 // [n_tokens, n_used]
@@ -311,6 +317,159 @@ __device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, cons
     }
 }
 
+// ---- a shared expert kept in Q8_0 -----------------------------------------------------------------
+// Its gate/up and down items sit in the slot the MXFP4 shared expert would take (first in grid
+// order) and hand their results over the same way; the arithmetic is that of the Q8_0 streaming
+// kernels (dsx_q8_0_kernels.hpp; crates/v4flash-kernels/kernels/shared_expert_fused.hip:69-199
+// computes the same products for the same purpose).  Tiles past sh_inter only count as done.
+// The lane's share of R weight rows against one activation row in LDS: the rows' blocks of a step
+// are all requested before the first is used, so that R times the bytes of a single row are in
+// flight (the streaming kernels' one-row loop is bound by the round trip of each step).
+template <int R>
+__device__ __forceinline__ void df_q8_rows_partial(float (&acc)[R], const uint8_t *const (&rows)[R],
+                                                   const uint8_t *lds_x, uint32_t n_blocks, uint32_t lane) {
+    for (uint32_t b0 = 0; b0 < n_blocks; b0 += 64u) {
+        const uint32_t b = b0 + lane;
+        const bool live = b < n_blocks;
+        const uint32_t bb = live ? b : n_blocks - 1u;  // clamped: the load stays in the row
+        U2A4 w[R][4];
+        uint16_t dbits[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint8_t *q = rows[r] + (size_t)n_blocks * 2u + (size_t)bb * 32u;
+            w[r][0] = gload8(q);
+            w[r][1] = gload8(q + 8u);
+            w[r][2] = gload8(q + 16u);
+            w[r][3] = gload8(q + 24u);
+            dbits[r] = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(rows[r] + (size_t)bb * 2u);
+        }
+        const uint4 x0 = *(const uint4 *)(lds_x + bb * 32u);
+        const uint4 x1 = *(const uint4 *)(lds_x + bb * 32u + 16u);
+        const float xs = *(const float *)(lds_x + n_blocks * 32u + bb * 4u);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float dw = live ? __half2float(__ushort_as_half(dbits[r])) : 0.0f;
+            int sum = 0;
+            sum = __builtin_amdgcn_sdot4((int)w[r][0].x, (int)x0.x, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][0].y, (int)x0.y, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][1].x, (int)x0.z, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][1].y, (int)x0.w, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][2].x, (int)x1.x, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][2].y, (int)x1.y, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][3].x, (int)x1.z, sum, false);
+            sum = __builtin_amdgcn_sdot4((int)w[r][3].y, (int)x1.w, sum, false);
+            acc[r] += dw * xs * (float)sum;   // the streaming kernels' arithmetic, term by term
+        }
+    }
+}
+
+__device__ __forceinline__ void df_q8_gate_up_item(const DecodeFusedParams &p, uint32_t t, uint32_t tile,
+                                                   uint8_t *lds) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t ms = t * p.n_slots + p.n_used, row0 = tile * 16u;
+    if (row0 < p.sh_inter) {
+        const uint32_t nb = p.hidden / 32u, row_bytes = q8_0_act_row_bytes(nb);
+        const uint8_t *xrow = p.xq8 + (uint64_t)t * p.xq8_row_bytes;
+        q8_0_stage(lds, 1u, row_bytes, tid, [&](uint32_t) { return xrow; });
+        __syncthreads();
+        const uint64_t wstride = (uint64_t)nb * 34u;
+        // the wave's four rows (wave, wave + 4, ...) two at a time, gate and up together
+#pragma unroll
+        for (uint32_t half = 0; half < 2u; half++) {
+            const uint32_t ra = row0 + wave + half * 8u, rb = ra + 4u;
+            const uint8_t *const rows[4] = {p.sh_gate + (uint64_t)ra * wstride, p.sh_up + (uint64_t)ra * wstride,
+                                            p.sh_gate + (uint64_t)rb * wstride, p.sh_up + (uint64_t)rb * wstride};
+            float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            df_q8_rows_partial<4>(a, rows, lds, nb, lane);
+            const float g0 = wave_sum_f32(a[0]), u0 = wave_sum_f32(a[1]);
+            const float g1 = wave_sum_f32(a[2]), u1 = wave_sum_f32(a[3]);
+            if (lane == 0) {
+                df_store_f32(p.mid + (uint64_t)ms * p.inter + ra, swiglu_clamp(g0, u0, p.sh_clamp, 1.0f));
+                df_store_f32(p.mid + (uint64_t)ms * p.inter + rb, swiglu_clamp(g1, u1, p.sh_clamp, 1.0f));
+            }
+        }
+    }
+    if (tid == 0) __hip_atomic_fetch_add(p.slot_done + ms, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Waits until the lane's four mid values at `src` are there (lanes with live == false hold
+// nothing); the wait is wave-uniform and bounded like every other one.
+__device__ __forceinline__ float4 df_wait_mid4(const DecodeFusedParams &p, const float *src, bool live,
+                                               uint32_t ms, uint32_t item) {
+    const uint32_t lane = threadIdx.x & 63u;
+    float4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) v = *(const float4 *)src;
+    auto missing = [&]() {
+        return live && (__float_as_uint(v.x) == kMidUnwritten || __float_as_uint(v.y) == kMidUnwritten ||
+                        __float_as_uint(v.z) == kMidUnwritten || __float_as_uint(v.w) == kMidUnwritten);
+    };
+    bool flag_seen = false;
+    for (uint32_t spin = 0; __builtin_amdgcn_ballot_w64(missing()) != 0ull; spin++) {
+        if (spin > p.spin_limit) {
+            if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusMidWaitExpired);
+            if (missing()) v = float4{0.f, 0.f, 0.f, 0.f};
+            break;
+        }
+        if (!flag_seen) {
+            const uint32_t *flag = p.ready + ((uint64_t)ms * kDfFan + (item % kDfFan)) * kDfFanStride;
+            uint32_t polls = 0;
+            while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u &&
+                   polls < p.spin_limit) {
+                polls++;
+                for (uint32_t z = 0; z < p.poll_sleep; z += 8u) __builtin_amdgcn_s_sleep(8);
+            }
+            flag_seen = true;
+        } else {
+            __builtin_amdgcn_s_sleep(16);
+        }
+        if (live) {
+            v.x = df_load_f32(src + 0);
+            v.y = df_load_f32(src + 1);
+            v.z = df_load_f32(src + 2);
+            v.w = df_load_f32(src + 3);
+        }
+    }
+    return v;
+}
+
+// Rows [row0, row0 + 16) of the wave: the mid row (sh_inter values) is quantized to a Q8_0
+// activation row in LDS by every item that needs it, then each row of down is one pass of the wave.
+// Returns the lane's row (lane % 16) of the 16 results.
+__device__ __forceinline__ float df_q8_down_rows(const DecodeFusedParams &p, uint32_t t, uint32_t row0,
+                                                 uint32_t item, uint8_t *lds) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t ms = t * p.n_slots + p.n_used;
+    const uint32_t nb = p.sh_inter / 32u, n256 = (p.sh_inter + 255u) / 256u;
+    const float *mrow = p.mid + (uint64_t)ms * p.inter;
+    for (uint32_t blk = wave; blk < n256; blk += (uint32_t)kDfWaves) {
+        const uint32_t idx = blk * 256u + lane * 4u;
+        const bool live = idx < p.sh_inter;
+        const float4 v = df_wait_mid4(p, mrow + idx, live, ms, item);
+        uint32_t pk;
+        float d8;
+        q8_0_quantize_lane4(v, pk, d8);
+        if (live) {
+            *(uint32_t *)(lds + idx) = pk;
+            if ((lane & 7u) == 0u) *(float *)(lds + p.sh_inter + (idx >> 5) * 4u) = d8;
+        }
+    }
+    __syncthreads();
+    const uint64_t wstride = (uint64_t)nb * 34u;
+    float own = 0.0f;
+    for (uint32_t rr = 0; rr < 16u; rr += 4u) {   // four rows at a time
+        const uint8_t *base = p.sh_down + (uint64_t)(row0 + rr) * wstride;
+        const uint8_t *const rows[4] = {base, base + wstride, base + 2u * wstride, base + 3u * wstride};
+        float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        df_q8_rows_partial<4>(a, rows, lds, nb, lane);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float v = wave_sum_f32(a[i]);
+            if ((lane & 15u) == rr + (uint32_t)i) own = v;
+        }
+    }
+    return own;
+}
+
 template <bool SHARE>
 __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint32_t item,
                                                 uint8_t *tiles, float *s_yd,
@@ -322,6 +481,11 @@ __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint
     const uint32_t slot = df_slot_of(order, p.n_used, p.n_slots);
     const uint32_t row0 = df_xcd_contiguous(j, p.gu_tiles) * 16u;
     df_stamp(p, item, 0);
+    if (p.sh_q8 && slot == p.n_used) {   // uniform
+        df_q8_gate_up_item(p, t, row0 / 16u, tiles);
+        df_stamp(p, item, 3);
+        return;
+    }
 
     // the token's staged row goes out first (see df_gate_up_core)
     const uint8_t *xrow = p.xq + (uint64_t)t * p.xq_row_bytes;
@@ -471,6 +635,13 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
     const bool last = order + 1u == p.n_slots;   // this item adds up the token's rows
     df_stamp(p, trace_id, 0);
 
+    if (p.sh_q8 && slot == p.n_used) {   // uniform
+        const float own = df_q8_down_rows(p, t, row0, item, tiles);
+        if (last) df_combine(p, t, row0, own, slot);
+        else if (lane < 16u) df_store_f32(p.partials + ((uint64_t)t * p.n_slots + slot) * p.hidden + row0 + lane, own);
+        df_stamp(p, trace_id, 3);
+        return;
+    }
     const uint8_t *down_e = p.sh_down;
     int e = -1;
     if (slot < p.n_used) {

@@ -428,6 +428,8 @@ struct FrontParams {
     uint32_t mode, n_group, topk_group;
     uint32_t n_tokens, n_sb, xp_row_bytes, n_fill, fill_value, route;
     uint32_t fp6;   // staged rows in the grouped GEMMs' format (FP6 planes, 384 bytes per super-block)
+    uint8_t *xq8;   // also the tokens as Q8_0 activation rows ([k i8][k/32 f32]), or null
+    uint32_t xq8_row_bytes;
 };
 
 __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParams p) {
@@ -460,6 +462,15 @@ __global__ __launch_bounds__(kRouterThreads) void k_layer_front(const FrontParam
                                       (float *)(row + (size_t)p.n_sb * kStaged6Bytes) + b);
         else
             quantize_block_to_staged(v, lane, row + (size_t)b * 512u, (float *)(row + (size_t)p.n_sb * 512u) + b);
+        if (p.xq8 != nullptr) {
+            // the same elements as a Q8_0 row, for a shared expert kept in Q8_0
+            uint32_t pk;
+            float d8;
+            q8_0_quantize_lane4(v, pk, d8);
+            uint8_t *r8 = p.xq8 + (uint64_t)t * p.xq8_row_bytes;
+            *(uint32_t *)(r8 + (size_t)b * 256u + lane * 4u) = pk;
+            if ((lane & 7u) == 0u) *(float *)(r8 + (size_t)p.n_sb * 256u + ((size_t)b * 8u + (lane >> 3)) * 4u) = d8;
+        }
         v = nxt;
     }
     if (p.sel_in != nullptr)

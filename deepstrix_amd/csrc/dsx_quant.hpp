@@ -178,4 +178,25 @@ __device__ __forceinline__ void quantize_block_to_staged6(float4 v, uint32_t lan
     if (lane == 0) *d_out = r.d;
 }
 
+// Q8_0 activation quantizer, four consecutive elements per lane, eight lanes per 32-element block
+// (crates/v4flash-kernels/kernels/q8_0_matvec.hip:150-177): d = max|x| / 127, q = rint(x / d).
+// All lanes of the wave take part (lanes without elements pass zeros).
+__device__ __forceinline__ void q8_0_quantize_lane4(float4 v, uint32_t &packed, float &d) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float xs[4] = {v.x, v.y, v.z, v.w};
+    packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int q = (int)rintf(xs[i] * id);
+        q = q > 127 ? 127 : q;
+        q = q < -128 ? -128 : q;
+        packed |= (uint32_t)(q & 0xFF) << (8 * i);
+    }
+}
+
 }  // namespace dsx

@@ -2,7 +2,8 @@
 intermediate size differs from the routed one (docs/v41/ARCH_SPEC.md:239,
 crates/v4flash-kernels/src/het/dispatch.rs:196-214) -- against the CPU oracle at every token
 count that takes a different path: one launch / per-stage decode, by-expert, grouped GEMM with
-the shared expert on the int8 GEMM."""
+the shared expert on the int8 GEMM.  Up to three tokens the Q8_0 shared expert is computed by items
+of the one-launch decode path, from four on by the dense kernels on a side stream."""
 import numpy as np
 import pytest
 
@@ -46,7 +47,7 @@ def _check(s, layer, hw, T, modes=(1,)):
         assert H.compare_stats(out, want)["max_over_max"] < REGRESSION, (T, mode)
 
 
-@pytest.mark.parametrize("T", [1, 5, 14, 16, 64, 130, 300])
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 14, 16, 64, 130, 300])
 def test_small_layer_with_q8_0_shared_expert_of_another_width(T):
     dw = H.device_weights(SMALL)
     layer = MoeLayer(dw, T)
@@ -79,7 +80,7 @@ def v3_layer():
     return MoeLayer(dw, 512), H.host_weights_from_device(V3, dw)
 
 
-@pytest.mark.parametrize("T", [1, 4, 64, 512])
+@pytest.mark.parametrize("T", [1, 2, 4, 64, 512])
 def test_v3_shape_with_q8_0_shared_expert(T, v3_layer):
     layer, hw = v3_layer
     _check(V3, layer, hw, T, modes=(1, 2) if T <= 14 else (1,))
@@ -120,3 +121,14 @@ def test_side_stream_shared_expert_under_graph_capture(T, v3_layer):
     layer.run(dx, dl, out=out)
     torch.cuda.synchronize()
     assert torch.equal(out, eager)
+
+
+@pytest.mark.parametrize("T", [1, 2, 5])
+def test_q8_0_shared_expert_wider_than_the_routed_ones(T):
+    """A shared expert wider than the routed experts cannot sit in the one-launch path's mid rows
+    (they are `inter` long): it stays with the dense kernels at every token count."""
+    s = H.Shape(1024, 256, 16, 4, sh_gate_fmt=FMT_Q8_0, sh_down_fmt=FMT_Q8_0, sh_inter=384,
+                router_mode=1, n_group=4, topk_group=2, route_scale=2.5, bias_sigma=0.01,
+                clamp=10.0, seed=1207)
+    layer = MoeLayer(H.device_weights(s), T)
+    _check(s, layer, H.host_weights(s), T, modes=(1, 2))
