@@ -322,47 +322,6 @@ __device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, cons
 // order) and hand their results over the same way; the arithmetic is that of the Q8_0 streaming
 // kernels (dsx_q8_0_kernels.hpp; crates/v4flash-kernels/kernels/shared_expert_fused.hip:69-199
 // computes the same products for the same purpose).  Tiles past sh_inter only count as done.
-// The lane's share of R weight rows against one activation row in LDS: the rows' blocks of a step
-// are all requested before the first is used, so that R times the bytes of a single row are in
-// flight (the streaming kernels' one-row loop is bound by the round trip of each step).
-template <int R>
-__device__ __forceinline__ void df_q8_rows_partial(float (&acc)[R], const uint8_t *const (&rows)[R],
-                                                   const uint8_t *lds_x, uint32_t n_blocks, uint32_t lane) {
-    for (uint32_t b0 = 0; b0 < n_blocks; b0 += 64u) {
-        const uint32_t b = b0 + lane;
-        const bool live = b < n_blocks;
-        const uint32_t bb = live ? b : n_blocks - 1u;  // clamped: the load stays in the row
-        U2A4 w[R][4];
-        uint16_t dbits[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const uint8_t *q = rows[r] + (size_t)n_blocks * 2u + (size_t)bb * 32u;
-            w[r][0] = gload8(q);
-            w[r][1] = gload8(q + 8u);
-            w[r][2] = gload8(q + 16u);
-            w[r][3] = gload8(q + 24u);
-            dbits[r] = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(rows[r] + (size_t)bb * 2u);
-        }
-        const uint4 x0 = *(const uint4 *)(lds_x + bb * 32u);
-        const uint4 x1 = *(const uint4 *)(lds_x + bb * 32u + 16u);
-        const float xs = *(const float *)(lds_x + n_blocks * 32u + bb * 4u);
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const float dw = live ? __half2float(__ushort_as_half(dbits[r])) : 0.0f;
-            int sum = 0;
-            sum = __builtin_amdgcn_sdot4((int)w[r][0].x, (int)x0.x, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][0].y, (int)x0.y, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][1].x, (int)x0.z, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][1].y, (int)x0.w, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][2].x, (int)x1.x, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][2].y, (int)x1.y, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][3].x, (int)x1.z, sum, false);
-            sum = __builtin_amdgcn_sdot4((int)w[r][3].y, (int)x1.w, sum, false);
-            acc[r] += dw * xs * (float)sum;   // the streaming kernels' arithmetic, term by term
-        }
-    }
-}
-
 __device__ __forceinline__ void df_q8_gate_up_item(const DecodeFusedParams &p, uint32_t t, uint32_t tile,
                                                    uint8_t *lds) {
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
@@ -379,10 +338,10 @@ __device__ __forceinline__ void df_q8_gate_up_item(const DecodeFusedParams &p, u
             const uint32_t ra = row0 + wave + half * 8u, rb = ra + 4u;
             const uint8_t *const rows[4] = {p.sh_gate + (uint64_t)ra * wstride, p.sh_up + (uint64_t)ra * wstride,
                                             p.sh_gate + (uint64_t)rb * wstride, p.sh_up + (uint64_t)rb * wstride};
-            float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            df_q8_rows_partial<4>(a, rows, lds, nb, lane);
-            const float g0 = wave_sum_f32(a[0]), u0 = wave_sum_f32(a[1]);
-            const float g1 = wave_sum_f32(a[2]), u1 = wave_sum_f32(a[3]);
+            float a[4][1] = {{0.0f}, {0.0f}, {0.0f}, {0.0f}};
+            q8_0_rows_partial<4, 1>(a, rows, lds, row_bytes, nb, lane);
+            const float g0 = wave_sum_f32(a[0][0]), u0 = wave_sum_f32(a[1][0]);
+            const float g1 = wave_sum_f32(a[2][0]), u1 = wave_sum_f32(a[3][0]);
             if (lane == 0) {
                 df_store_f32(p.mid + (uint64_t)ms * p.inter + ra, swiglu_clamp(g0, u0, p.sh_clamp, 1.0f));
                 df_store_f32(p.mid + (uint64_t)ms * p.inter + rb, swiglu_clamp(g1, u1, p.sh_clamp, 1.0f));
@@ -459,11 +418,11 @@ __device__ __forceinline__ float df_q8_down_rows(const DecodeFusedParams &p, uin
     for (uint32_t rr = 0; rr < 16u; rr += 4u) {   // four rows at a time
         const uint8_t *base = p.sh_down + (uint64_t)(row0 + rr) * wstride;
         const uint8_t *const rows[4] = {base, base + wstride, base + 2u * wstride, base + 3u * wstride};
-        float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        df_q8_rows_partial<4>(a, rows, lds, nb, lane);
+        float a[4][1] = {{0.0f}, {0.0f}, {0.0f}, {0.0f}};
+        q8_0_rows_partial<4, 1>(a, rows, lds, 0u, nb, lane);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float v = wave_sum_f32(a[i]);
+            const float v = wave_sum_f32(a[i][0]);
             if ((lane & 15u) == rr + (uint32_t)i) own = v;
         }
     }

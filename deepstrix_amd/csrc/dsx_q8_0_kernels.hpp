@@ -6,11 +6,12 @@
 // exact in int32 (v_dot4_i32_i8), scaled by f16(d_w) * xscale in f32
 // (crates/v4flash-kernels/kernels/q8_0_matvec.hip:64-104).
 //
-// A wave reads one weight row front to back: lane l takes blocks l, l + 64, ... (32 int8 =
+// A wave reads weight rows front to back: lane l takes blocks l, l + 64, ... (32 int8 =
 // 32 contiguous bytes per lane, 2 KiB contiguous per wave load step), multiplies them with
 // the matching activation blocks of every token column (LDS), and the 64 partial sums of a
 // (row, column) are added by a butterfly.  A workgroup of four waves owns 16 rows, four per
-// wave.  These are streaming kernels for few columns (decode and small batches).
+// wave, which the wave streams together.  These are streaming kernels for few columns (decode
+// and small batches).
 #pragma once
 
 #include <hip/hip_fp16.h>
@@ -48,38 +49,51 @@ struct Q8Params {
     uint32_t n_sub;
 };
 
-// The lane's share of `row . x[c]` for NT columns, over all of its blocks.
-template <int NT>
-__device__ __forceinline__ void q8_0_row_partial(float (&acc)[NT], const uint8_t *__restrict__ row,
-                                                 const uint8_t *lds_x, uint32_t col_stride,
-                                                 uint32_t n_blocks, uint32_t lane) {
-    const uint8_t *quants = row + (size_t)n_blocks * 2u;
+// The lane's share of `rows[r] . x[c]` for R weight rows and NT columns, over all of its blocks.  The
+// rows' blocks of a step are all requested before the first is used, so that R times the bytes of a
+// single row are in flight: one row at a time is bound by the round trip of each step (a row of 64
+// blocks is a single step; a decode step's shared expert went from 69 to 54 us with four rows).
+// Per (row, column) the sum runs over the lane's blocks in ascending order, one term
+// f16(d_w) * xscale * int32 dot per block.
+template <int R, int NT>
+__device__ __forceinline__ void q8_0_rows_partial(float (&acc)[R][NT], const uint8_t *const (&rows)[R],
+                                                  const uint8_t *lds_x, uint32_t col_stride,
+                                                  uint32_t n_blocks, uint32_t lane) {
     for (uint32_t b0 = 0; b0 < n_blocks; b0 += 64u) {
         const uint32_t b = b0 + lane;
         const bool live = b < n_blocks;
         const uint32_t bb = live ? b : n_blocks - 1u;  // clamped: the load stays in the row
-        const U2A4 w0 = gload8(quants + (size_t)bb * 32u);
-        const U2A4 w1 = gload8(quants + (size_t)bb * 32u + 8u);
-        const U2A4 w2 = gload8(quants + (size_t)bb * 32u + 16u);
-        const U2A4 w3 = gload8(quants + (size_t)bb * 32u + 24u);
-        const uint16_t dbits = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(row + (size_t)bb * 2u);
-        const float dw = live ? __half2float(__ushort_as_half(dbits)) : 0.0f;
+        U2A4 w[R][4];
+        uint16_t dbits[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint8_t *q = rows[r] + (size_t)n_blocks * 2u + (size_t)bb * 32u;
+            w[r][0] = gload8(q);
+            w[r][1] = gload8(q + 8u);
+            w[r][2] = gload8(q + 16u);
+            w[r][3] = gload8(q + 24u);
+            dbits[r] = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(rows[r] + (size_t)bb * 2u);
+        }
 #pragma unroll
         for (int c = 0; c < NT; c++) {
             const uint8_t *xc = lds_x + (size_t)c * col_stride;
             const uint4 x0 = *(const uint4 *)(xc + bb * 32u);
             const uint4 x1 = *(const uint4 *)(xc + bb * 32u + 16u);
             const float xs = *(const float *)(xc + n_blocks * 32u + bb * 4u);
-            int s = 0;
-            s = __builtin_amdgcn_sdot4((int)w0.x, (int)x0.x, s, false);
-            s = __builtin_amdgcn_sdot4((int)w0.y, (int)x0.y, s, false);
-            s = __builtin_amdgcn_sdot4((int)w1.x, (int)x0.z, s, false);
-            s = __builtin_amdgcn_sdot4((int)w1.y, (int)x0.w, s, false);
-            s = __builtin_amdgcn_sdot4((int)w2.x, (int)x1.x, s, false);
-            s = __builtin_amdgcn_sdot4((int)w2.y, (int)x1.y, s, false);
-            s = __builtin_amdgcn_sdot4((int)w3.x, (int)x1.z, s, false);
-            s = __builtin_amdgcn_sdot4((int)w3.y, (int)x1.w, s, false);
-            acc[c] += dw * xs * (float)s;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const float dw = live ? __half2float(__ushort_as_half(dbits[r])) : 0.0f;
+                int s = 0;
+                s = __builtin_amdgcn_sdot4((int)w[r][0].x, (int)x0.x, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][0].y, (int)x0.y, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][1].x, (int)x0.z, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][1].y, (int)x0.w, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][2].x, (int)x1.x, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][2].y, (int)x1.y, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][3].x, (int)x1.z, s, false);
+                s = __builtin_amdgcn_sdot4((int)w[r][3].y, (int)x1.w, s, false);
+                acc[r][c] += dw * xs * (float)s;
+            }
         }
     }
 }
@@ -161,18 +175,27 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_gate_up(const Q8Params p
     __syncthreads();
 
     const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
-    for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
-        const uint32_t row = row0 + r;
-        float g[NT], u[NT];
+    // the wave's four rows (wave, wave + 4, ...) two at a time, gate and up together
+    static_assert(kQ8RowsPerWg == 4 * kQ8Waves, "four rows per wave");
 #pragma unroll
-        for (int c = 0; c < NT; c++) g[c] = u[c] = 0.0f;
-        q8_0_row_partial<NT>(g, g_e + (uint64_t)row * wstride, lds_x, row_bytes, p.n_blocks, lane);
-        q8_0_row_partial<NT>(u, u_e + (uint64_t)row * wstride, lds_x, row_bytes, p.n_blocks, lane);
+    for (uint32_t half = 0; half < 2u; half++) {
+        const uint32_t ra = row0 + wave + half * 2u * kQ8Waves, rb = ra + kQ8Waves;
+        const uint8_t *const rows[4] = {g_e + (uint64_t)ra * wstride, u_e + (uint64_t)ra * wstride,
+                                        g_e + (uint64_t)rb * wstride, u_e + (uint64_t)rb * wstride};
+        float a[4][NT];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int c = 0; c < NT; c++) a[r][c] = 0.0f;
+        q8_0_rows_partial<4, NT>(a, rows, lds_x, row_bytes, p.n_blocks, lane);
 #pragma unroll
         for (int c = 0; c < NT; c++) {
-            const float gs = wave_sum_f32(g[c]), us = wave_sum_f32(u[c]);
-            if (lane == 0 && (uint32_t)c < cnt)
-                p.dst[(uint64_t)s_dest[c] * p.n_rows + row] = swiglu_clamp(gs, us, clamp, s_ew[c]);
+            const float g0 = wave_sum_f32(a[0][c]), u0 = wave_sum_f32(a[1][c]);
+            const float g1 = wave_sum_f32(a[2][c]), u1 = wave_sum_f32(a[3][c]);
+            if (lane == 0 && (uint32_t)c < cnt) {
+                p.dst[(uint64_t)s_dest[c] * p.n_rows + ra] = swiglu_clamp(g0, u0, clamp, s_ew[c]);
+                p.dst[(uint64_t)s_dest[c] * p.n_rows + rb] = swiglu_clamp(g1, u1, clamp, s_ew[c]);
+            }
         }
     }
 }
@@ -193,24 +216,28 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_decode(const Q8Para
                [&](uint32_t j) { return p.xq + (uint64_t)j * p.x_stride; });
     __syncthreads();
     const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
-    for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
-        const uint32_t row = row0 + r;
-        float total = 0.0f;
-        for (uint32_t s = 0; s < n_slots; s++) {
-            const uint8_t *w;
-            if (s < p.n_used) {
-                const int e = s_sel[s];
-                if (e < 0) continue;
-                w = p.w0 + (uint64_t)e * p.bpe0;
-            } else {
-                w = p.sh_w0;
-            }
-            float a[1] = {0.0f};
-            q8_0_row_partial<1>(a, w + (uint64_t)row * wstride, lds_x + (size_t)s * row_bytes, row_bytes,
-                                p.n_blocks, lane);
-            total += wave_sum_f32(a[0]);
+    // the wave's four rows (wave, wave + 4, ...) at once, slot after slot
+    float total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t s = 0; s < n_slots; s++) {
+        const uint8_t *w;
+        if (s < p.n_used) {
+            const int e = s_sel[s];
+            if (e < 0) continue;
+            w = p.w0 + (uint64_t)e * p.bpe0;
+        } else {
+            w = p.sh_w0;
         }
-        if (lane == 0) p.dst[row] = total;
+        const uint8_t *base = w + (uint64_t)(row0 + wave) * wstride;
+        const uint8_t *const rows[4] = {base, base + kQ8Waves * wstride, base + 2u * kQ8Waves * wstride,
+                                        base + 3u * kQ8Waves * wstride};
+        float a[4][1] = {{0.0f}, {0.0f}, {0.0f}, {0.0f}};
+        q8_0_rows_partial<4, 1>(a, rows, lds_x + (size_t)s * row_bytes, row_bytes, p.n_blocks, lane);
+#pragma unroll
+        for (int r = 0; r < 4; r++) total[r] += wave_sum_f32(a[r][0]);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) p.dst[row0 + wave + (uint32_t)r * kQ8Waves] = total[r];
     }
 }
 
@@ -245,18 +272,24 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_by_expert(const Q8P
     __syncthreads();
     const uint8_t *w_e = (p.sh_w0 != nullptr && e >= p.n_expert) ? p.sh_w0 : p.w0 + (uint64_t)e * p.bpe0;
     const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
-    for (uint32_t r = wave; r < (uint32_t)kQ8RowsPerWg; r += kQ8Waves) {
-        const uint32_t row = row0 + r;
-        float a[NT];
+    // the wave's four rows (wave, wave + 4, ...) at once
+    const uint8_t *base = w_e + (uint64_t)(row0 + wave) * wstride;
+    const uint8_t *const rows[4] = {base, base + kQ8Waves * wstride, base + 2u * kQ8Waves * wstride,
+                                    base + 3u * kQ8Waves * wstride};
+    float a[4][NT];
 #pragma unroll
-        for (int c = 0; c < NT; c++) a[c] = 0.0f;
-        q8_0_row_partial<NT>(a, w_e + (uint64_t)row * wstride, lds_x, row_bytes, p.n_blocks, lane);
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int c = 0; c < NT; c++) a[r][c] = 0.0f;
+    q8_0_rows_partial<4, NT>(a, rows, lds_x, row_bytes, p.n_blocks, lane);
+#pragma unroll
+    for (int r = 0; r < 4; r++)
 #pragma unroll
         for (int c = 0; c < NT; c++) {
-            const float v = wave_sum_f32(a[c]);
-            if (lane == 0 && (uint32_t)c < cnt) p.dst[(uint64_t)s_dest[c] * p.n_rows + row] = v;
+            const float v = wave_sum_f32(a[r][c]);
+            if (lane == 0 && (uint32_t)c < cnt)
+                p.dst[(uint64_t)s_dest[c] * p.n_rows + row0 + wave + (uint32_t)r * kQ8Waves] = v;
         }
-    }
 }
 
 // ---- host side ----------------------------------------------------------------------------
