@@ -474,9 +474,12 @@ struct Q8GemmParams {
     float clamp, sh_clamp;
 };
 
-inline size_t q8_0_gemm_lds_bytes(uint32_t n_blocks, bool pair) {
+// columns (double buffered) | activation scales | the waves' weight chunks (double buffered) | the
+// rows' block scales of two chunks at a time (double buffered): 72 KB with both matrices, so that
+// two workgroups share a CU
+inline size_t q8_0_gemm_lds_bytes(bool pair) {
     const uint32_t m = pair ? 2u : 1u;
-    return kQgAOff + (size_t)kQgWaves * m * 4096u + (size_t)m * kQgRows * n_blocks * 2u;
+    return kQgAOff + (size_t)kQgWaves * m * 4096u + (size_t)2u * m * kQgRows * 16u;
 }
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
@@ -527,14 +530,10 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
     wbase[0] = (extra ? p.sh_w0 : p.w0 + (uint64_t)e * p.bpe0) + (uint64_t)(rt * kQgRows) * row_bytes;
     if (PAIR) wbase[M - 1] = (extra ? p.sh_w1 : p.w1 + (uint64_t)e * p.bpe1) + (uint64_t)(rt * kQgRows) * row_bytes;
 
-    // the 64 rows' block scales of each matrix, once: dw[matrix][row][block]
+    // the rows' block scales travel with the chunks: 16 bytes per row hold the scales of two chunks
+    // (8 blocks), fetched by one instruction per matrix every other chunk (wave mm: lane -> row)
     const uint32_t dw_off = kQgAOff + kQgWaves * M * 4096u;
-    uint16_t *s_dw = (uint16_t *)(smem + dw_off);
-    for (uint32_t i = tid; i < M * (uint32_t)kQgRows * nb; i += kQgWaves * 64u) {
-        const uint32_t mm = i / ((uint32_t)kQgRows * nb), j = i - mm * (uint32_t)kQgRows * nb;
-        const uint32_t r = j / nb, b = j - r * nb;
-        s_dw[i] = *(const DSX_GLOBAL uint16_t *)(uintptr_t)(wbase[PAIR ? mm : 0] + (uint64_t)r * row_bytes + b * 2u);
-    }
+    const uint8_t *s_dw = smem + dw_off;   // [buffer][matrix][row][16 B]
     __syncthreads();  // s_src visible
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
@@ -550,6 +549,9 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
         b_fetch[ii] = s_src[wave * 32u + ii * 8u + l8] * p.act_row_bytes + c8 * 16u;
     // activation scales: waves 0 and 1, lane -> column 64 w + lane, the chunk's 4 floats
     const uint32_t xs_lds = __builtin_amdgcn_readfirstlane(lds0 + kQgXsOff + (wave & 1u) * 1024u);
+    const uint32_t dw_lds = __builtin_amdgcn_readfirstlane(lds0 + dw_off);
+    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint8_t *dw_base = (M == 2u && wave_u == 1u) ? wbase[M - 1] : wbase[0];   // wave mm fetches matrix mm's
     const uint32_t xs_fetch = s_src[(wave & 1u) * 64u + lane] * p.act_row_bytes + nb * 32u;
     const bool b_live = wave * 32u < cnt;
     auto issue = [&](uint32_t c, uint32_t buf) {
@@ -565,6 +567,10 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
                 lds_dma16(b_lds + buf * 16384u + (uint32_t)ii * 1024u, p.act, b_fetch[ii] + c * 128u);
         }
         if (wave < 2u) lds_dma16(xs_lds + buf * 2048u, p.act, xs_fetch + c * 16u);
+        // (a last, single chunk reads 8 bytes past the scales, into the row's own quants)
+        if ((c & 1u) == 0u && wave_u < M)
+            lds_dma16(dw_lds + ((c >> 1) & 1u) * (M * kQgRows * 16u) + wave_u * (kQgRows * 16u), dw_base,
+                      lane * row_bytes + (c >> 1) * 16u);
     };
 
     // read side: lane (row / column n16, 8-byte piece g4 of a block's 32 bytes)
@@ -597,7 +603,8 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
         for (uint32_t mm = 0; mm < M; mm++) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const uint2 h = *(const uint2 *)(s_dw + (size_t)(mm * kQgRows + wave * 16u + g4 * 4u + q) * nb + c * 4u);
+                const uint2 h = *(const uint2 *)(s_dw + ((size_t)((c >> 1) & 1u) * M + mm) * (kQgRows * 16u) +
+                                                 (size_t)(wave * 16u + g4 * 4u + q) * 16u + (c & 1u) * 8u);
                 dw[mm][q][0] = __half2float(__ushort_as_half((uint16_t)(h.x & 0xFFFFu)));
                 dw[mm][q][1] = __half2float(__ushort_as_half((uint16_t)(h.x >> 16)));
                 dw[mm][q][2] = __half2float(__ushort_as_half((uint16_t)(h.y & 0xFFFFu)));
@@ -654,8 +661,8 @@ __global__ __launch_bounds__(kQgWaves * 64) void k_q8_0_gemm(const Q8GemmParams 
 
 // Raised once per device by the library's set-up, with the device current.
 inline void q8_0_gemm_raise_lds_limits() {
-    (void)hipFuncSetAttribute((const void *)k_q8_0_gemm<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
-    (void)hipFuncSetAttribute((const void *)k_q8_0_gemm<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gemm<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+    (void)hipFuncSetAttribute((const void *)k_q8_0_gemm<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
 }
 
 template <bool PAIR>
@@ -666,8 +673,7 @@ inline int q8_0_gemm(hipStream_t st, const Q8GemmParams &p, uint32_t max_wi) {
     const uint64_t act_rows = (uint64_t)p.n_tokens * (p.n_used + 1u);
     if ((uint64_t)p.n_rows * p.n_blocks * 34u > 0xFFFFFFFFull || act_rows * p.act_row_bytes > 0xFFFFFFFFull)
         return q8_0_fail(DSX_ERR_INVALID_ARG, "q8_0 gemm", "a weight matrix or the activation rows exceed 4 GiB");
-    const size_t lds = q8_0_gemm_lds_bytes(p.n_blocks, PAIR);
-    if (lds > 140 * 1024) return q8_0_fail(DSX_ERR_UNSUPPORTED, "q8_0 gemm", "k too large for the scale table in LDS");
+    const size_t lds = q8_0_gemm_lds_bytes(PAIR);
     const uint32_t per_xcd = (max_wi + 7u) / 8u;
     const uint64_t grid = (uint64_t)8u * per_xcd * p.n_row_tiles;
     if (grid > 0x7FFFFFFFull) return q8_0_fail(DSX_ERR_INVALID_ARG, "q8_0 gemm", "grid too large");
