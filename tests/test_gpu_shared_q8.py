@@ -86,12 +86,13 @@ def test_v3_shape_with_q8_0_shared_expert(T, v3_layer):
     _check(V3, layer, hw, T, modes=(1, 2) if T <= 14 else (1,))
 
 
-@pytest.mark.parametrize("T", [2, 4, 12])
+@pytest.mark.parametrize("T", [2, 4, 12, 24, 130])
 def test_side_stream_shared_expert_under_graph_capture(T, v3_layer):
-    """From two tokens on, the one-launch decode path computes the Q8_0 shared expert on a stream
-    of its own, forked from and joined to the caller's: a capture of the caller's stream must
-    record both branches, and every replay must give what the eager call gives -- bitwise, with
-    the program's own work and synchronizations between the replays."""
+    """From four tokens on (decode, by-expert and GEMM paths alike) the Q8_0 shared expert is
+    computed on a stream of its own, forked from and joined to the caller's: a capture of the
+    caller's stream must record both branches, and every replay must give what the eager call
+    gives -- bitwise, with the program's own work and synchronizations between the replays.
+    (Two tokens: the shared expert inside the decode launch, no second stream.)"""
     s = V3
     layer, hw = v3_layer
     layer.set_decode(fused=1)
