@@ -371,7 +371,30 @@ def main():
         extra[f"us_per_token_T{T}"] = (time.perf_counter() - t1) * 1e6 / reps / T
 
     if not args.no_prefill:
-        extra["prefill_T4096"] = prefill_leg(layers[0].w, base, H, torch, np)
+        # on the engine's rows (the layout a checkpoint loads into) and on the planar form of the
+        # same matrices (rewritten in place once after loading; identical results): the planar
+        # figures are the leg's own, the other layout's time is quoted beside them
+        on_rows = prefill_leg(layers[0].w, base, H, torch, np)
+        dwp = H.device_weights(H.Shape(**base.__dict__), planar=True)
+        pre = prefill_leg(dwp, base, H, torch, np)
+        pre["weights_layout"] = ("planar (DSX_FMT_MXFP4_PLANAR: nibble blocks and scales in separate planes, "
+                                 "made in place by dsx_mxfp4_rows_to_planar)")
+        pre["ms_per_layer_engine_rows"] = on_rows["ms_per_layer"]
+        pre["tokens_per_s_engine_rows"] = on_rows["tokens_per_s"]
+        extra["prefill_T4096"] = pre
+        # the decode step on planar weights, rotating over as many layers as the headline figure
+        del dwp
+        lps = [MoeLayer(H.device_weights(H.Shape(**{**base.__dict__, "seed": base.seed + 0x100 * i}), planar=True), 1)
+               for i in range(L)]
+        for i in range(W):
+            lps[i % L].run(x_all[i:i + 1], lg_all[i:i + 1], out=out)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(W, W + K):
+            lps[i % L].run(x_all[i:i + 1], lg_all[i:i + 1], out=out)
+        torch.cuda.synchronize()
+        extra["us_per_token_T1_planar_weights"] = (time.perf_counter() - t1) * 1e6 / K
+        del lps
     if not args.no_chain:
         extra["chain_8_layers_T2"] = chain_leg(H, torch, np)
     if not args.no_extra:

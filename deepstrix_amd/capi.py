@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(PKG, "lib", "libdsx_moe.so")
 
 FMT_Q8_0 = 8
 FMT_MXFP4 = 39
+FMT_MXFP4_PLANAR = 1039  # the same matrix with nibble blocks and scales in separate planes (include/dsx_moe.h)
 SRC_F32, SRC_BF16, SRC_F8E4M3 = 0, 1, 2  # dsx_q8_0_weights_from_hf source types
 ROUTER_SQRT_SOFTPLUS, ROUTER_SIGMOID, ROUTER_SOFTMAX = 0, 1, 2
 ERR_INVALID_ARG, ERR_SHAPE, ERR_UNSUPPORTED, ERR_DEVICE = -1, -2, -3, -4
@@ -78,6 +79,8 @@ SIGNATURES = {
     "dsx_mxfp4_repack_hf_to_v2": (_int, [_vp, _vp, _vp, _vp, _u32, _u32]),
     "dsx_q8_0_weights_from_hf": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32]),
     "dsx_q8_0_repack_rows": (_int, [_vp, _vp, _vp, _u32, _u32]),
+    "dsx_mxfp4_rows_to_planar": (_int, [_vp, _vp, _u32, _u32, _u32, _u64]),
+    "dsx_mxfp4_planar_to_rows": (_int, [_vp, _vp, _u32, _u32, _u32, _u64]),
     "dsx_dequant_rows": (_int, [_vp, _int, _vp, _vp, _u32, _u32]),
     "dsx_moe_layer_create": (_int, [C.POINTER(LayerDesc), C.POINTER(_vp)]),
     "dsx_moe_layer_destroy": (None, [_vp]),

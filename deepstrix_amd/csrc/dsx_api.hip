@@ -91,10 +91,18 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_decode_fused<0, false>);
         allow_lds(k_mxfp4_decode_fused<8, true>);
         allow_lds(k_mxfp4_decode_fused<0, true>);
+        allow_lds(k_mxfp4_decode_fused<8, false, true>);
+        allow_lds(k_mxfp4_decode_fused<0, false, true>);
+        allow_lds(k_mxfp4_decode_fused<8, true, true>);
+        allow_lds(k_mxfp4_decode_fused<0, true, true>);
         allow_lds(k_mxfp4_gemm<true, kGemmMT>);
         allow_lds(k_mxfp4_gemm<false, kGemmMT>);
         allow_lds(k_mxfp4_gemm<true, kGemmMTNarrow>);
         allow_lds(k_mxfp4_gemm<false, kGemmMTNarrow>);
+        allow_lds(k_mxfp4_gemm<true, kGemmMT, true>);
+        allow_lds(k_mxfp4_gemm<false, kGemmMT, true>);
+        allow_lds(k_mxfp4_relayout<true>);
+        allow_lds(k_mxfp4_relayout<false>);
         allow_lds(k_mxfp4_down_decode<false>);
         allow_lds(k_mxfp4_down_decode<true>);
         allow_lds(k_mxfp4_down_decode<true, 9>);
@@ -170,8 +178,9 @@ int group_build_big(hipStream_t st, int32_t *group_count, int32_t *group_offset,
 
 // Grouped GEMM launch; max_wi bounds the number of work items, MT is the chunk they were built
 // with (kGemmMT or kGemmMTNarrow).
+// planar: the weights are in the planar form (wide tile only).
 template <bool PAIR, int MT = kGemmMT>
-int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
+int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi, bool planar = false) {
     if (max_wi == 0) return DSX_OK;
     const uint32_t per_xcd = (max_wi + 7u) / 8u;
     const uint64_t grid = (uint64_t)8u * per_xcd * p.n_row_tiles;
@@ -181,6 +190,15 @@ int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi) {
     if ((uint64_t)p.n_rows * p.n_sb * kSuperBytes > 0xFFFFFFFFull ||
         act_rows * p.act_row_bytes > 0xFFFFFFFFull)
         return fail(DSX_ERR_INVALID_ARG, "gemm: a weight matrix or the activation rows exceed 4 GiB");
+    if constexpr (MT == kGemmMT) {
+        if (planar) {
+            hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT, true>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
+                               gemm_lds_bytes(MT), st, p);
+            return launched(PAIR ? "gate_up gemm" : "down gemm");
+        }
+    } else if (planar) {
+        return fail(DSX_ERR_UNSUPPORTED, "gemm: the narrow tile reads the engine's row layout only");
+    }
     hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
                        gemm_lds_bytes(MT), st, p);
     return launched(PAIR ? "gate_up gemm" : "down gemm");
@@ -331,7 +349,8 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
     if (dtype == DSX_FMT_Q8_0)
         return q8_0_gate_up_decode(st, mid, gate, up, xq, ew, selected, sh_gate, sh_up, sh_clamp,
                                    gbpe, ubpe, n_used, clamp, n_rows, n_blocks);
-    if (dtype != DSX_FMT_MXFP4)
+    const bool planar = dtype == DSX_FMT_MXFP4_PLANAR;
+    if (dtype != DSX_FMT_MXFP4 && !planar)
         return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_batch: no kernel for dtype %d", dtype);
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_gate_up_batch: n_rows=%u must be a multiple of 16", n_rows);
@@ -347,6 +366,7 @@ static int gate_up_decode_impl(hipStream_t st, int dtype, float *mid, const uint
     p.sh_gate = sh_gate; p.sh_up = sh_up; p.gbpe = gbpe; p.ubpe = ubpe; p.n_used = n_used;
     p.chunk = 1; p.clamp = clamp; p.sh_clamp = sh_clamp; p.n_rows = n_rows; p.n_blocks = n_blocks;
     p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
+    p.planar = planar ? 1u : 0u;
     const uint32_t n_slots = n_used + (sh_gate ? 1u : 0u);
     if (staged) {
         if (n_rows % 256 != 0 || !midp || !aligned(xq, 16))
@@ -383,7 +403,8 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     if (dtype == DSX_FMT_Q8_0)
         return q8_0_down_decode(st, out, down, xq, selected, sh_down, dbpe, xq_slot_stride, n_used,
                                 n_rows, n_blocks_in);
-    if (dtype != DSX_FMT_MXFP4)
+    const bool planar = dtype == DSX_FMT_MXFP4_PLANAR;
+    if (dtype != DSX_FMT_MXFP4 && !planar)
         return fail(DSX_ERR_UNSUPPORTED, "moe_down_batched: no kernel for dtype %d", dtype);
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_down_batched: n_rows=%u must be a multiple of 16", n_rows);
@@ -403,7 +424,7 @@ static int down_decode_impl(hipStream_t st, int dtype, float *out, const uint8_t
     p.out = out; p.down = down; p.xq = xq; p.selected = selected; p.sh_down = sh_down;
     p.residual = residual;
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.n_slots = n_slots;
-    p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
+    p.n_rows = n_rows; p.n_blocks_in = n_blocks_in; p.planar = planar ? 1u : 0u;
     // two workgroups of 8 waves per CU, all resident at once and of equal size where the row
     // count allows (7168 rows on 256 CUs: 512 workgroups of 14 rows)
     const uint32_t even = (n_rows + 2u * g_num_cu - 1u) / (2u * g_num_cu);
@@ -480,7 +501,8 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
                                       expert_members, work_items, n_work_items, max_work_items,
                                       gbpe, ubpe, n_used, chunk, clamp, n_rows, n_blocks, sh_gate, sh_up,
                                       sh_clamp, n_expert, n_tokens);
-    if (dtype != DSX_FMT_MXFP4)
+    const bool planar = dtype == DSX_FMT_MXFP4_PLANAR;
+    if (dtype != DSX_FMT_MXFP4 && !planar)
         return fail(DSX_ERR_UNSUPPORTED, "moe_gate_up_chunked_rows: no kernel for dtype %d", dtype);
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: n_rows=%u must be a multiple of 16", n_rows);
@@ -505,7 +527,7 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     p.n_rows = n_rows; p.n_blocks = n_blocks;
     p.xq_row_bytes = staged ? staged_row_bytes(n_blocks) : n_blocks * kQ8kBytes;
     p.sh_gate = sh_gate; p.sh_up = sh_up; p.sh_clamp = sh_clamp; p.n_expert = n_expert; p.n_tokens = n_tokens;
-    p.n_sub = n_sub;
+    p.n_sub = n_sub; p.planar = planar ? 1u : 0u;
     hipStream_t st = S(stream);
     switch (nt) {
         case 1: launch_gate_up_be<1>(st, p, max_work_items, lds, staged); break;
@@ -549,7 +571,8 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
                                    expert_members, work_items, n_work_items, max_work_items, dbpe,
                                    xq_slot_stride, n_used, chunk, n_rows, n_blocks_in, sh_down, n_expert,
                                    n_tokens);
-    if (dtype != DSX_FMT_MXFP4)
+    const bool planar = dtype == DSX_FMT_MXFP4_PLANAR;
+    if (dtype != DSX_FMT_MXFP4 && !planar)
         return fail(DSX_ERR_UNSUPPORTED, "moe_down_by_expert: no kernel for dtype %d", dtype);
     if (n_rows == 0 || n_rows % 16 != 0)
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: n_rows=%u must be a multiple of 16", n_rows);
@@ -576,7 +599,7 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
     p.dbpe = dbpe; p.xq_slot_stride = xq_slot_stride; p.n_used = n_used; p.chunk = chunk;
     p.n_rows = n_rows; p.n_blocks_in = n_blocks_in;
     p.sh_down = sh_down; p.n_expert = n_expert; p.n_tokens = n_tokens;
-    p.n_sub = n_sub;
+    p.n_sub = n_sub; p.planar = planar ? 1u : 0u;
     hipStream_t st = S(stream);
     switch (nt) {
         case 1: launch_down_be<1>(st, p, max_work_items, lds, staged); break;
@@ -691,6 +714,44 @@ int dsx_mxfp4_repack_hf_to_v2(dsx_stream_t stream, uint8_t *dst, const uint8_t *
     hipLaunchKernelGGL(k_mxfp4_repack, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, S(stream),
                        dst, packed, scale, out, nb);
     return launched("mxfp4_repack");
+}
+
+static int mxfp4_relayout(hipStream_t st, bool to_planar, uint8_t *w, uint32_t n_rows, uint32_t cols,
+                          uint32_t n_matrices, uint64_t stride) {
+    const char *who = to_planar ? "mxfp4_rows_to_planar" : "mxfp4_planar_to_rows";
+    if (n_matrices == 0 || n_rows == 0 || cols == 0) return DSX_OK;
+    if (!w) return fail(DSX_ERR_INVALID_ARG, "%s: null pointer", who);
+    if (n_rows % 16 != 0 || cols % 256 != 0)
+        return fail(DSX_ERR_SHAPE, "%s: n_rows=%u must be a multiple of 16, cols=%u of 256", who, n_rows, cols);
+    const uint32_t n_sb = cols / 256;
+    const uint64_t mat_bytes = (uint64_t)n_rows * n_sb * kSuperBytes;
+    if (stride < mat_bytes || stride % 8 != 0 || !aligned(w, 8))
+        return fail(DSX_ERR_SHAPE, "%s: matrices must be 8-byte aligned and at least %llu bytes apart", who,
+                    (unsigned long long)mat_bytes);
+    const size_t lds = (size_t)16 * n_sb * kSuperBytes;   // one 16-row tile
+    if (lds > kLdsBudget)
+        return fail(DSX_ERR_UNSUPPORTED, "%s: cols=%u: a 16-row tile exceeds LDS", who, cols);
+    if (int rc_init = need_init(who)) return rc_init;
+    for (uint32_t m0 = 0; m0 < n_matrices; m0 += 65535u) {
+        const uint32_t m = std::min(65535u, n_matrices - m0);
+        uint8_t *first = w + (uint64_t)m0 * stride;
+        if (to_planar)
+            hipLaunchKernelGGL(k_mxfp4_relayout<true>, dim3(n_rows / 16, m), dim3(256), lds, st, first, n_sb, stride);
+        else
+            hipLaunchKernelGGL(k_mxfp4_relayout<false>, dim3(n_rows / 16, m), dim3(256), lds, st, first, n_sb, stride);
+        if (int rc = launched(who)) return rc;
+    }
+    return DSX_OK;
+}
+
+int dsx_mxfp4_rows_to_planar(dsx_stream_t stream, uint8_t *w, uint32_t n_rows, uint32_t cols,
+                             uint32_t n_matrices, uint64_t stride) {
+    return mxfp4_relayout(S(stream), true, w, n_rows, cols, n_matrices, stride);
+}
+
+int dsx_mxfp4_planar_to_rows(dsx_stream_t stream, uint8_t *w, uint32_t n_rows, uint32_t cols,
+                             uint32_t n_matrices, uint64_t stride) {
+    return mxfp4_relayout(S(stream), false, w, n_rows, cols, n_matrices, stride);
 }
 
 int dsx_q8_0_weights_from_hf(dsx_stream_t stream, uint8_t *dst, const void *src,

@@ -204,7 +204,7 @@ struct DfListCols {
 // of the item's list), SwiGLU, write-through store of the mid values, the slots' counters.
 // PRE: the single column's staged row was requested by the caller before the weights (ex0..3,
 // early_yd) -- loads of a wave return in order, so the row must not queue behind them.
-template <int NT, bool PRE, typename Cols>
+template <int NT, bool PRE, bool PLANAR, typename Cols>
 __device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, const Cols c,
                                                 uint32_t n, const uint8_t *gate_e,
                                                 const uint8_t *up_e, float clamp, uint32_t row0,
@@ -214,18 +214,18 @@ __device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, cons
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     constexpr uint32_t kStep = kDfWaves * 64u;
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    const uint64_t row_stride = (uint64_t)p.n_sb * kSuperBytes;
-    const uint8_t *grow = gate_e + (uint64_t)(row0 + r) * row_stride;
-    const uint8_t *urow = up_e + (uint64_t)(row0 + r) * row_stride;
+    constexpr uint32_t kStepW = PLANAR ? 128u : (uint32_t)kSuperBytes;
+    const WRow grow = w_row(gate_e, row0 + r, p.n_sb, PLANAR);
+    const WRow urow = w_row(up_e, row0 + r, p.n_sb, PLANAR);
     uint32_t sb = wave;
     WSuper g0, u0, g1, u1;
     {
         const uint32_t last = p.n_sb - 1u;
         const uint32_t b0 = sb < last ? sb : last, b1 = sb + kDfWaves < last ? sb + kDfWaves : last;
-        g0 = load_wsuper(grow + (uint64_t)b0 * kSuperBytes, kb);
-        u0 = load_wsuper(urow + (uint64_t)b0 * kSuperBytes, kb);
-        g1 = load_wsuper(grow + (uint64_t)b1 * kSuperBytes, kb);
-        u1 = load_wsuper(urow + (uint64_t)b1 * kSuperBytes, kb);
+        g0 = load_wsuper(grow, (uint64_t)(b0) * kStepW, kb);
+        u0 = load_wsuper(urow, (uint64_t)(b0) * kStepW, kb);
+        g1 = load_wsuper(grow, (uint64_t)(b1) * kStepW, kb);
+        u1 = load_wsuper(urow, (uint64_t)(b1) * kStepW, kb);
     }
 
     if (PRE) {
@@ -264,14 +264,14 @@ __device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, cons
     while (sb + 3 * kDfWaves < p.n_sb) {
         compute(sb, g0, u0);
         DSX_AFTER_PRODUCTS();
-        g0 = load_wsuper(grow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
-        u0 = load_wsuper(urow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
+        g0 = load_wsuper(grow, (uint64_t)((sb + 2 * kDfWaves)) * kStepW, kb);
+        u0 = load_wsuper(urow, (uint64_t)((sb + 2 * kDfWaves)) * kStepW, kb);
         DSX_PIN();
         asm volatile("" : "+v"(g1.s.x), "+v"(g1.s.y), "+v"(u1.s.x), "+v"(u1.s.y));
         compute(sb + kDfWaves, g1, u1);
         DSX_AFTER_PRODUCTS();
-        g1 = load_wsuper(grow + (uint64_t)(sb + 3 * kDfWaves) * kSuperBytes, kb);
-        u1 = load_wsuper(urow + (uint64_t)(sb + 3 * kDfWaves) * kSuperBytes, kb);
+        g1 = load_wsuper(grow, (uint64_t)((sb + 3 * kDfWaves)) * kStepW, kb);
+        u1 = load_wsuper(urow, (uint64_t)((sb + 3 * kDfWaves)) * kStepW, kb);
         DSX_PIN();
         sb += 2 * kDfWaves;
     }
@@ -279,8 +279,8 @@ __device__ __forceinline__ void df_gate_up_core(const DecodeFusedParams &p, cons
         WSuper g2 = {}, u2 = {};
         const bool third = sb + 2 * kDfWaves < p.n_sb;
         if (third) {
-            g2 = load_wsuper(grow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
-            u2 = load_wsuper(urow + (uint64_t)(sb + 2 * kDfWaves) * kSuperBytes, kb);
+            g2 = load_wsuper(grow, (uint64_t)((sb + 2 * kDfWaves)) * kStepW, kb);
+            u2 = load_wsuper(urow, (uint64_t)((sb + 2 * kDfWaves)) * kStepW, kb);
         }
         DSX_PIN();
         compute(sb, g0, u0);
@@ -429,7 +429,7 @@ __device__ __forceinline__ float df_q8_down_rows(const DecodeFusedParams &p, uin
     return own;
 }
 
-template <bool SHARE>
+template <bool SHARE, bool PLANAR>
 __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint32_t item,
                                                 uint8_t *tiles, float *s_yd,
                                                 float (*s_red)[2][4][64], DfCols *cols) {
@@ -474,7 +474,7 @@ __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint
     const DfPair pr = df_pair<SHARE>(p, t, slot, e);
     if (pr.cnt == 0u) return;   // the token above serves this one
     if (pr.cnt == 1u) {
-        df_gate_up_core<1, true>(p, DfOneCol{t, t * p.n_slots + slot, pr.ew0}, 1u, gate_e, up_e, clamp, row0,
+        df_gate_up_core<1, true, PLANAR>(p, DfOneCol{t, t * p.n_slots + slot, pr.ew0}, 1u, gate_e, up_e, clamp, row0,
                                  tiles, s_yd, s_red, ex0, ex1, ex2, ex3, early_yd, item);
     } else if (SHARE) {
         // the pair's two columns in one pass over the tile's weights
@@ -483,7 +483,7 @@ __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint
             cols->tok[1] = pr.t1; cols->ms[1] = pr.ms1; cols->ew[1] = pr.ew1;
         }
         __syncthreads();
-        df_gate_up_core<2, false>(p, DfListCols{cols, 0u}, 2u, gate_e, up_e, clamp, row0, tiles, s_yd,
+        df_gate_up_core<2, false, PLANAR>(p, DfListCols{cols, 0u}, 2u, gate_e, up_e, clamp, row0, tiles, s_yd,
                                   s_red, ex0, ex1, ex2, ex3, early_yd, item);
     }
     df_stamp(p, item, 3);
@@ -578,7 +578,7 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
 
 // NSB > 0: inter / 256 == NSB, straight-line code with all NSB super-blocks of the wave's rows in
 // registers; NSB == 0: any inter, in passes of up to 8 super-blocks.
-template <int NSB, bool SHARE>
+template <int NSB, bool SHARE, bool PLANAR>
 __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_t item,
                                              uint8_t *tiles, float *s_yd) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -625,7 +625,8 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
     float4 mv0 = *(const float4 *)(mrow0 + (size_t)blk0 * 256u + lane * 4u);
     float4 mv1 = *(const float4 *)(mrow0 + (size_t)blk1 * 256u + lane * 4u);
 
-    const uint8_t *wrow = down_e + (uint64_t)(row0 + r) * nsb * kSuperBytes;
+    constexpr uint32_t kStepW = PLANAR ? 128u : (uint32_t)kSuperBytes;
+    const WRow wrow = w_row(down_e, row0 + r, nsb, PLANAR);
     constexpr int kHold = NSB > 0 ? NSB : 8;
     WSuper w[kHold];
     // the first part of what this wave will read goes out now, the rest once the mid row is
@@ -633,7 +634,7 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
     const int early = (int)p.dn_early;
 #pragma unroll
     for (int b = 0; b < kHold; b++)
-        if ((NSB > 0 || (uint32_t)b < nsb) && b < early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
+        if ((NSB > 0 || (uint32_t)b < nsb) && b < early) w[b] = load_wsuper(wrow, (uint64_t)(b) * kStepW, kb);
 
     const DfPair pr = df_pair<SHARE>(p, t, slot, e);
     const uint32_t cnt = pr.cnt;
@@ -695,7 +696,7 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
             // the mid row is there: the rest of the weights goes out
 #pragma unroll
             for (int b = 0; b < kHold; b++)
-                if ((NSB > 0 || (uint32_t)b < nsb) && b >= early) w[b] = load_wsuper(wrow + (uint64_t)b * kSuperBytes, kb);
+                if ((NSB > 0 || (uint32_t)b < nsb) && b >= early) w[b] = load_wsuper(wrow, (uint64_t)(b) * kStepW, kb);
             df_stamp(p, trace_id, 1);
         }
         uint8_t *tl = tiles + (size_t)c * nsb * 512u;
@@ -736,7 +737,7 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
             WSuper w2[8];
 #pragma unroll
             for (int b = 0; b < 8; b++)
-                if (b0 + b < nsb) w2[b] = load_wsuper(wrow + (uint64_t)(b0 + b) * kSuperBytes, kb);
+                if (b0 + b < nsb) w2[b] = load_wsuper(wrow, (uint64_t)((b0 + b)) * kStepW, kb);
 #pragma unroll
             for (int b = 0; b < 8; b++) {
                 if (b0 + b < nsb) {
@@ -777,7 +778,7 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
 }
 
 // LDS (dynamic): max(n_sb (twice that when tokens share experts), n_sb_in) tiles of 512 bytes | as many floats
-template <int NSB, bool SHARE>
+template <int NSB, bool SHARE, bool PLANAR = false>
 __global__ __launch_bounds__(kDfWaves * 64, 1) void k_mxfp4_decode_fused(const DecodeFusedParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[kDfWaves][2][4][64];
@@ -788,11 +789,11 @@ __global__ __launch_bounds__(kDfWaves * 64, 1) void k_mxfp4_decode_fused(const D
     uint8_t *tiles = smem;
     float *s_yd = (float *)(smem + (size_t)n_max * 512u);
     if (blockIdx.x < p.n_gu_items)
-        df_gate_up_item<SHARE>(p, blockIdx.x, tiles, s_yd, s_red, &s_cols);
+        df_gate_up_item<SHARE, PLANAR>(p, blockIdx.x, tiles, s_yd, s_red, &s_cols);
     else if (blockIdx.x == p.n_gu_items)
         df_relay_item(p);
     else
-        df_down_item<NSB, SHARE>(p, blockIdx.x - p.n_gu_items - 1u, tiles, s_yd);
+        df_down_item<NSB, SHARE, PLANAR>(p, blockIdx.x - p.n_gu_items - 1u, tiles, s_yd);
 }
 
 }  // namespace dsx

@@ -212,6 +212,45 @@ __device__ __forceinline__ WSuper load_wsuper(const uint8_t *__restrict__ row_su
     return w;
 }
 
+// ---- where a matrix keeps a row's super-blocks ------------------------------------------------
+// The engine's rows hold each super-block's 128 nibble bytes and 8 scale bytes together (136
+// bytes, so a block starts on a cache line only every 16th time).  The planar form permutes the
+// bytes of every 16-row tile within the tile: first the 16 rows' nibble blocks, row-major at
+// 128 bytes per super-block -- every block is one whole cache line -- then the tile's scales
+// as [super-block][row in tile][8 bytes], so that the scales a 16-row fragment needs of one
+// super-block are one line too.  A tile keeps its place and size (16 n_sb 136 bytes, a multiple
+// of 128), so whoever streams whole tiles reads the same stretch of memory in either form, and
+// consecutive super-blocks of a row are `w_step` bytes apart in nibbles and scales alike.
+struct WRow {
+    const uint8_t *nib, *sc;
+};
+__device__ __forceinline__ uint32_t w_step(bool planar) { return planar ? 128u : (uint32_t)kSuperBytes; }
+// byte offsets, from the start of the matrix, of a row's first nibble block and first scale group
+__device__ __forceinline__ void w_row_offsets(uint32_t row, uint32_t n_sb, bool planar, uint64_t &nib,
+                                              uint64_t &sc) {
+    if (planar) {
+        const uint64_t tile = (uint64_t)(row >> 4) * n_sb * (16u * kSuperBytes);
+        nib = tile + (row & 15u) * n_sb * 128u;
+        sc = tile + n_sb * 2048u + (row & 15u) * 8u;
+    } else {
+        nib = (uint64_t)row * n_sb * kSuperBytes;
+        sc = nib + 128u;
+    }
+}
+__device__ __forceinline__ WRow w_row(const uint8_t *mat, uint32_t row, uint32_t n_sb, bool planar) {
+    uint64_t nib, sc;
+    w_row_offsets(row, n_sb, planar, nib, sc);
+    return WRow{mat + nib, mat + sc};
+}
+// super-block at byte offset `off` (= index x w_step) of the row
+__device__ __forceinline__ WSuper load_wsuper(const WRow &w, uint64_t off, uint32_t kb) {
+    WSuper r;
+    r.a0 = gload16(w.nib + off + kb * 16u);
+    r.a1 = gload16(w.nib + off + 64u + kb * 16u);
+    r.s = gload8(w.sc + off);
+    return r;
+}
+
 __device__ __forceinline__ v8i b_operand(const uint8_t *tile, uint32_t off0, uint32_t off1) {
     const uint4 lo = *(const uint4 *)(tile + off0);
     const uint4 hi = *(const uint4 *)(tile + off1);

@@ -127,6 +127,7 @@ struct GateUpParams {
     // by-expert: a work item of `chunk` members is served by n_sub workgroups along grid.y,
     // NT columns each (0 is read as 1)
     uint32_t n_sub;
+    uint32_t planar;  // the matrices are in the planar form (dsx_device.hpp)
 };
 
 // LDS: [n_blocks] tiles of 512 * NT bytes | yd[n_blocks * NT] floats
@@ -227,9 +228,9 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
 
     // ---- the first two super-blocks of weights go out before anything else -----------
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    const uint64_t row_stride = (uint64_t)p.n_blocks * kSuperBytes;
-    const uint8_t *grow = gate_e + (uint64_t)(row0 + r) * row_stride;
-    const uint8_t *urow = up_e + (uint64_t)(row0 + r) * row_stride;
+    const uint32_t wstep = w_step(p.planar != 0u);
+    const WRow grow = w_row(gate_e, row0 + r, p.n_blocks, p.planar != 0u);
+    const WRow urow = w_row(up_e, row0 + r, p.n_blocks, p.planar != 0u);
     uint32_t sb = wave;
     // The first two loads are unconditional as well (a wave without a block of its own reads
     // the row's last one and never uses it), so that the k loop starts from a known count of
@@ -238,10 +239,10 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     {
         const uint32_t last = p.n_blocks - 1u;
         const uint32_t b0 = sb < last ? sb : last, b1 = sb + kGuWaves < last ? sb + kGuWaves : last;
-        g0 = load_wsuper(grow + (uint64_t)b0 * kSuperBytes, kb);
-        u0 = load_wsuper(urow + (uint64_t)b0 * kSuperBytes, kb);
-        g1 = load_wsuper(grow + (uint64_t)b1 * kSuperBytes, kb);
-        u1 = load_wsuper(urow + (uint64_t)b1 * kSuperBytes, kb);
+        g0 = load_wsuper(grow, (uint64_t)(b0) * wstep, kb);
+        u0 = load_wsuper(urow, (uint64_t)(b0) * wstep, kb);
+        g1 = load_wsuper(grow, (uint64_t)(b1) * wstep, kb);
+        u1 = load_wsuper(urow, (uint64_t)(b1) * wstep, kb);
     }
 
     // ---- activations into LDS -----------------------------------------------------------
@@ -293,15 +294,15 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
     while (sb + 3 * kGuWaves < p.n_blocks) {
         compute(sb, g0, u0);
         DSX_AFTER_PRODUCTS();
-        g0 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
-        u0 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+        g0 = load_wsuper(grow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
+        u0 = load_wsuper(urow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
         DSX_PIN();
         // (the scale bytes of the second pair are not touched before this point either)
         asm volatile("" : "+v"(g1.s.x), "+v"(g1.s.y), "+v"(u1.s.x), "+v"(u1.s.y));
         compute(sb + kGuWaves, g1, u1);
         DSX_AFTER_PRODUCTS();
-        g1 = load_wsuper(grow + (uint64_t)(sb + 3 * kGuWaves) * kSuperBytes, kb);
-        u1 = load_wsuper(urow + (uint64_t)(sb + 3 * kGuWaves) * kSuperBytes, kb);
+        g1 = load_wsuper(grow, (uint64_t)((sb + 3 * kGuWaves)) * wstep, kb);
+        u1 = load_wsuper(urow, (uint64_t)((sb + 3 * kGuWaves)) * wstep, kb);
         DSX_PIN();
         sb += 2 * kGuWaves;
     }
@@ -311,8 +312,8 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         WSuper g2 = {}, u2 = {};
         const bool third = sb + 2 * kGuWaves < p.n_blocks;
         if (third) {
-            g2 = load_wsuper(grow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
-            u2 = load_wsuper(urow + (uint64_t)(sb + 2 * kGuWaves) * kSuperBytes, kb);
+            g2 = load_wsuper(grow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
+            u2 = load_wsuper(urow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
         }
         DSX_PIN();
         compute(sb, g0, u0);
@@ -407,6 +408,7 @@ struct DownDecodeParams {
     uint64_t dbpe;
     uint32_t xq_slot_stride, n_used, n_slots, n_rows, n_blocks_in;
     uint32_t rows_per_wg;     // output rows of one workgroup, at most 16: the grid is sized to fill the CUs evenly
+    uint32_t planar;          // the matrices are in the planar form (dsx_device.hpp)
 };
 
 // LDS: [n_slots * n_blocks_in] tiles of 512 bytes | yd[n_slots * n_blocks_in]
@@ -436,7 +438,12 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     // rows of the 16-row fragment past the workgroup's share (or the matrix) repeat its last
     // row: every lane loads, so no load sits behind a condition, and their sums are not stored
     const uint32_t n_live = min(p.rows_per_wg, p.n_rows - row0);
-    const uint64_t row_off = (uint64_t)(row0 + min(r, n_live - 1u)) * nb * kSuperBytes;
+    // the lane's row inside a matrix: offsets of its nibble blocks and of its scales
+    const bool planar = p.planar != 0u;
+    const uint32_t wstep = w_step(planar);
+    const uint32_t wrow_i = row0 + min(r, n_live - 1u);
+    uint64_t row_off, sc_off;
+    w_row_offsets(wrow_i, nb, planar, row_off, sc_off);
     // blockIdx.y = token: its picks, its n_slots activation rows, its output row
     const int32_t *selected = p.selected + (uint64_t)blockIdx.y * p.n_used;
     const uint8_t *xq = p.xq + (uint64_t)blockIdx.y * p.n_slots * p.xq_slot_stride;
@@ -448,9 +455,9 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
         const int e = (slot < p.n_used) ? selected[slot] : 0;
         const uint8_t *base = (slot < p.n_used) ? p.down + (uint64_t)(e < 0 ? 0 : e) * p.dbpe
                                                 : p.sh_down;
-        return base + (uint64_t)b * kSuperBytes;
+        return base + (uint64_t)b * wstep;
     };
-    auto unit_ptr = [&](uint32_t un) -> const uint8_t * { return unit_base(un) + row_off; };
+    auto unit_w = [&](const uint8_t *ub) -> WRow { return WRow{ub + row_off, ub + sc_off}; };
     // With a fixed unit count the addresses of the later units are worked out here, while the
     // picks can still be read through the scalar cache (after the first asm statement below the
     // compiler reads them with vector loads, and waiting for one of those waits for every
@@ -494,17 +501,17 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     uint32_t un = wave;
     WSuper w0 = {}, w1 = {}, w2 = {}, w3 = {}, w4 = {};
     if (NU > 0) {
-        w0 = load_wsuper(unit_ptr(un), kb);
-        if (NU > 1) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
-        if (NU > 2) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
-        if (NU > 3) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
-        if (NU > 4) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
+        w0 = load_wsuper(unit_w(unit_base(un)), 0u, kb);
+        if (NU > 1) w1 = load_wsuper(unit_w(unit_base(un + kDownWaves)), 0u, kb);
+        if (NU > 2) w2 = load_wsuper(unit_w(unit_base(un + 2 * kDownWaves)), 0u, kb);
+        if (NU > 3) w3 = load_wsuper(unit_w(unit_base(un + 3 * kDownWaves)), 0u, kb);
+        if (NU > 4) w4 = load_wsuper(unit_w(unit_base(un + 4 * kDownWaves)), 0u, kb);
     } else {
-        if (un < units) w0 = load_wsuper(unit_ptr(un), kb);
-        if (un + kDownWaves < units) w1 = load_wsuper(unit_ptr(un + kDownWaves), kb);
-        if (un + 2 * kDownWaves < units) w2 = load_wsuper(unit_ptr(un + 2 * kDownWaves), kb);
-        if (un + 3 * kDownWaves < units) w3 = load_wsuper(unit_ptr(un + 3 * kDownWaves), kb);
-        if (un + 4 * kDownWaves < units) w4 = load_wsuper(unit_ptr(un + 4 * kDownWaves), kb);
+        if (un < units) w0 = load_wsuper(unit_w(unit_base(un)), 0u, kb);
+        if (un + kDownWaves < units) w1 = load_wsuper(unit_w(unit_base(un + kDownWaves)), 0u, kb);
+        if (un + 2 * kDownWaves < units) w2 = load_wsuper(unit_w(unit_base(un + 2 * kDownWaves)), 0u, kb);
+        if (un + 3 * kDownWaves < units) w3 = load_wsuper(unit_w(unit_base(un + 3 * kDownWaves)), 0u, kb);
+        if (un + 4 * kDownWaves < units) w4 = load_wsuper(unit_w(unit_base(un + 4 * kDownWaves)), 0u, kb);
     }
 
     if (tid < p.n_slots) s_sel[tid] = (tid < p.n_used) ? sel_mine : 0;
@@ -545,7 +552,7 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     if (I < NU) {                                                                            \
         compute(un + I * kDownWaves, W);                                                     \
         asm volatile("" : "+v"(acc) :: "memory");                                            \
-        if (I + 5 < NU) W = load_wsuper(later[I + 5 < NU ? I : 0] + row_off, kb);            \
+        if (I + 5 < NU) W = load_wsuper(unit_w(later[I + 5 < NU ? I : 0]), 0u, kb);            \
         asm volatile("" ::: "memory");                                                       \
     }
         DSX_DOWN_STEP(0, w0)
@@ -568,7 +575,7 @@ __global__ __launch_bounds__(kDownWaves * 64) void k_mxfp4_down_decode(const Dow
     } else {
 #define DSX_DOWN_STEP(W)                                                                     \
     compute(un, W);                                                                          \
-    if (un + 5 * kDownWaves < units) W = load_wsuper(unit_ptr(un + 5 * kDownWaves), kb);     \
+    if (un + 5 * kDownWaves < units) W = load_wsuper(unit_w(unit_base(un + 5 * kDownWaves)), 0u, kb);     \
     un += kDownWaves;                                                                        \
     if (un >= units) break;
         while (un < units) {
@@ -611,6 +618,7 @@ struct DownByExpertParams {
     const uint8_t *sh_down;  // the extra expert (index n_expert, slot n_used), or null
     uint32_t n_expert, n_tokens;
     uint32_t n_sub;  // workgroups along grid.y per work item, NT columns each (0 is read as 1)
+    uint32_t planar; // the matrices are in the planar form (dsx_device.hpp)
 };
 
 // LDS: [n_blocks_in] tiles of 512 * NT bytes | yd[n_blocks_in * NT]
@@ -647,12 +655,12 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     }
 
     const uint32_t r = lane & 15u, kb = lane >> 4;
-    const uint8_t *wrow = (extra ? p.sh_down : p.down + (uint64_t)e * p.dbpe) +
-                          (uint64_t)(row0 + r) * nb * kSuperBytes;
+    const uint32_t wstep = w_step(p.planar != 0u);
+    const WRow wrow = w_row(extra ? p.sh_down : p.down + (uint64_t)e * p.dbpe, row0 + r, nb, p.planar != 0u);
     uint32_t sb = wave;
     WSuper w0 = {}, w1 = {};
-    if (sb < nb) w0 = load_wsuper(wrow + (uint64_t)sb * kSuperBytes, kb);
-    if (sb + kDownBeWaves < nb) w1 = load_wsuper(wrow + (uint64_t)(sb + kDownBeWaves) * kSuperBytes, kb);
+    if (sb < nb) w0 = load_wsuper(wrow, (uint64_t)(sb) * wstep, kb);
+    if (sb + kDownBeWaves < nb) w1 = load_wsuper(wrow, (uint64_t)((sb + kDownBeWaves)) * wstep, kb);
 
     __syncthreads();
     if (STAGED) {
@@ -676,11 +684,11 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     };
     while (sb < nb) {
         compute(sb, w0);
-        if (sb + 2 * kDownBeWaves < nb) w0 = load_wsuper(wrow + (uint64_t)(sb + 2 * kDownBeWaves) * kSuperBytes, kb);
+        if (sb + 2 * kDownBeWaves < nb) w0 = load_wsuper(wrow, (uint64_t)((sb + 2 * kDownBeWaves)) * wstep, kb);
         sb += kDownBeWaves;
         if (sb >= nb) break;
         compute(sb, w1);
-        if (sb + 2 * kDownBeWaves < nb) w1 = load_wsuper(wrow + (uint64_t)(sb + 2 * kDownBeWaves) * kSuperBytes, kb);
+        if (sb + 2 * kDownBeWaves < nb) w1 = load_wsuper(wrow, (uint64_t)((sb + 2 * kDownBeWaves)) * wstep, kb);
         sb += kDownBeWaves;
     }
 

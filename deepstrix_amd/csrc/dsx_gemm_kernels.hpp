@@ -77,7 +77,7 @@ __device__ __forceinline__ uint32_t gemm_dest_row(uint32_t m, uint32_t n_tokens,
 // accumulators and of the column LDS, so that two workgroups share a CU (the second template
 // argument of the launch bounds asks for four waves per SIMD) -- with few members per group the
 // kernel only streams weights, and two workgroups keep twice the weight loads in flight.
-template <bool PAIR, int MT>
+template <bool PAIR, int MT, bool PLANAR = false>
 __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp4_gemm(const GemmParams p) {
     constexpr int kGemmCG = MT / 16;                    // column groups
     constexpr int kGemmHalfBytes = gemm_half_bytes(MT);  // half a super-block of all columns in LDS
@@ -118,7 +118,11 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     const uint32_t wi = (uint32_t)p.work_items[item];
     const uint32_t e = wi >> 16, start = wi & 0xFFFFu;
     const bool extra = e >= p.n_expert;
-    const uint32_t row_stride = p.n_sb * kSuperBytes;
+    // (PLANAR: the matrices in the planar form of dsx_device.hpp -- every 128-byte piece of a
+    // row that a lane group fetches is then one whole cache line instead of parts of two)
+    constexpr uint32_t kStepW = PLANAR ? 128u : (uint32_t)kSuperBytes;
+    const uint32_t row_stride = p.n_sb * kStepW;           // between the rows of a 16-row tile
+    const uint32_t tile_row = p.n_sb * kSuperBytes;        // a sixteenth of a tile, in either form
     const uint8_t *wbase[2];
     uint32_t row0[2];
     if (PAIR) {
@@ -147,9 +151,11 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
         for (int m = 0; m < 2; m++)
-            a_slab[r][m] = __builtin_amdgcn_readfirstlane((row0[m] + wave * kRowsPerWave + r * 16u) * row_stride);
-    // scales: one instruction per row set, lane -> (row lane / 2 of the wave's 32, dword lane % 2)
-    const uint32_t sc_fetch = (lane >> 1) * row_stride + 128u + (lane & 1u) * 4u;
+            a_slab[r][m] = __builtin_amdgcn_readfirstlane((row0[m] + wave * kRowsPerWave + r * 16u) * tile_row);
+    // scales: one instruction per row set, lane -> (row lane / 2 of the wave's 32, dword lane % 2);
+    // planar: the 128 bytes of each of the wave's two 16-row tiles, behind the tile's nibble blocks
+    const uint32_t sc_fetch = PLANAR ? (lane >> 5) * 16u * tile_row + p.n_sb * 2048u + (lane & 31u) * 4u
+                                     : (lane >> 1) * row_stride + 128u + (lane & 1u) * 4u;
     // The part of an address that all lanes share (row set, fragment, super-block) goes into the
     // scalar base of the load; the lane's own offset is the same register for every weight load.
     auto issue_a = [&](uint32_t sb) {
@@ -160,10 +166,10 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
 #pragma unroll
                 for (int i = 0; i < 2; i++)
                     lds_dma16(a_lds + (uint32_t)((r * 2 + m) * 2048 + i * 1024),
-                              wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kSuperBytes), a_fetch);
+                              wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kStepW), a_fetch);
 #pragma unroll
         for (int m = 0; m < 2; m++)
-            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kSuperBytes), sc_fetch);
+            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kStepW), sc_fetch);
     };
     issue_a(0);
 
@@ -199,10 +205,10 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         if (L < 4 * kGemmRF) {
             const int f = L >> 1, i = L & 1, r = f >> 1, m = f & 1;
             lds_dma16(a_lds + (uint32_t)(f * 2048 + i * 1024),
-                      wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kSuperBytes), a_fetch);
+                      wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kStepW), a_fetch);
         } else {
             const int m = L - 4 * kGemmRF;
-            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kSuperBytes), sc_fetch);
+            lds_dma4(a_lds + kScaleOff + (uint32_t)m * 256u, wbase[m] + (a_slab[0][m] + sb * kStepW), sc_fetch);
         }
     };
     constexpr int kAFirst = 8;  // of them requested during the first half of a super-block

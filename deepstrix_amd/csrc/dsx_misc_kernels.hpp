@@ -1033,6 +1033,35 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
     }
 }
 
+// MXFP4 matrices between the engine's rows (136-byte super-blocks) and the planar form
+// (dsx_device.hpp), in place: the permutation stays inside each 16-row tile, so a workgroup
+// reads one tile (grid.x) of one matrix (grid.y) into LDS and writes it back in the other
+// order, 8 bytes per thread and step.  TO_PLANAR picks the direction.
+// LDS (dynamic): 16 n_sb 136 bytes
+template <bool TO_PLANAR>
+__global__ __launch_bounds__(256) void k_mxfp4_relayout(uint8_t *__restrict__ w, uint32_t n_sb,
+                                                        uint64_t stride) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t tile_bytes = 16u * n_sb * kSuperBytes, n_pieces = tile_bytes / 8u;
+    uint8_t *tile = w + (uint64_t)blockIdx.y * stride + (uint64_t)blockIdx.x * tile_bytes;
+    for (uint32_t i = threadIdx.x; i < n_pieces; i += 256u) *(uint2 *)(smem + i * 8u) = *(const uint2 *)(tile + i * 8u);
+    __syncthreads();
+    const uint32_t n_nib = 16u * n_sb * 16u;   // 8-byte pieces of nibbles
+    for (uint32_t i = threadIdx.x; i < n_pieces; i += 256u) {
+        // piece i of the planar order sits at rows_off in the row order
+        uint32_t rows_off;
+        if (i < n_nib) {
+            const uint32_t blk = i >> 4, row = blk / n_sb, sb = blk - row * n_sb;
+            rows_off = (row * n_sb + sb) * kSuperBytes + (i & 15u) * 8u;
+        } else {
+            const uint32_t s = i - n_nib, sb = s >> 4, row = s & 15u;
+            rows_off = (row * n_sb + sb) * kSuperBytes + 128u;
+        }
+        if (TO_PLANAR) *(uint2 *)(tile + i * 8u) = *(const uint2 *)(smem + rows_off);
+        else *(uint2 *)(tile + rows_off) = *(const uint2 *)(smem + i * 8u);
+    }
+}
+
 // HF packed nibbles + E8M0 scales -> v2 super-block rows, one thread per 32-element block.
 // crates/v4flash-kernels/kernels/mxfp4_repack.hip:35-65 (same bytes as
 // crates/v4flash-core/src/hf_v41.rs:1208-1232).

@@ -19,7 +19,7 @@ from typing import Optional
 import torch
 
 from . import capi
-from .capi import FMT_MXFP4, FMT_Q8_0, check, lib
+from .capi import FMT_MXFP4, FMT_MXFP4_PLANAR, FMT_Q8_0, check, lib
 
 
 def _stream() -> int:
@@ -189,6 +189,19 @@ def q8_0_repack_rows(dst, src, num_rows, blocks_per_row):
     check(lib().dsx_q8_0_repack_rows(_stream(), _p(dst), _p(src), num_rows, blocks_per_row))
 
 
+def mxfp4_rows_to_planar(w, n_rows, cols, n_matrices=1, stride=None):
+    """MXFP4 matrices in the engine's rows -> the planar form, in place (include/dsx_moe.h)."""
+    capi.init()
+    stride = n_rows * (cols // 256) * 136 if stride is None else stride
+    check(lib().dsx_mxfp4_rows_to_planar(_stream(), _p(w), n_rows, cols, n_matrices, stride))
+
+
+def mxfp4_planar_to_rows(w, n_rows, cols, n_matrices=1, stride=None):
+    capi.init()
+    stride = n_rows * (cols // 256) * 136 if stride is None else stride
+    check(lib().dsx_mxfp4_planar_to_rows(_stream(), _p(w), n_rows, cols, n_matrices, stride))
+
+
 def dequant_rows(dt, y, rows, n_rows, cols):
     capi.init()
     check(lib().dsx_dequant_rows(_stream(), dt, _p(y), _p(rows), n_rows, cols))
@@ -196,7 +209,7 @@ def dequant_rows(dt, y, rows, n_rows, cols):
 
 def matrix_bytes(fmt: int, rows: int, cols: int) -> int:
     """bytes_per_expert for one matrix (crates/v4flash-kernels/src/weight_contract.rs:146-158)."""
-    if fmt == FMT_MXFP4:
+    if fmt in (FMT_MXFP4, FMT_MXFP4_PLANAR):
         return rows * (cols // 256) * 136
     if fmt == FMT_Q8_0:
         return rows * (cols // 32) * 34

@@ -12,8 +12,8 @@ from typing import Optional
 import torch
 
 from . import capi
-from .capi import FMT_MXFP4, LayerDesc, check, lib
-from .dispatch import matrix_bytes
+from .capi import FMT_MXFP4, FMT_MXFP4_PLANAR, LayerDesc, check, lib
+from .dispatch import matrix_bytes, mxfp4_rows_to_planar
 
 
 @dataclass
@@ -49,6 +49,24 @@ class LayerWeights:
     norm_w: Optional[torch.Tensor] = None
     norm_eps: float = 1e-6
     router_w: Optional[torch.Tensor] = None
+
+
+    def to_planar(self) -> "LayerWeights":
+        """Rewrites every MXFP4 tensor in place into the planar form (FMT_MXFP4_PLANAR: same bytes
+        in another order, same results; the grouped GEMMs read it faster) and returns self."""
+        def conv(t, fmt, rows, cols, n):
+            if fmt != FMT_MXFP4:
+                return fmt
+            mxfp4_rows_to_planar(t, rows, cols, n)
+            return FMT_MXFP4_PLANAR
+        self.gate_fmt = conv(self.gate, self.gate_fmt, self.inter, self.hidden, self.n_expert)
+        self.up_fmt = conv(self.up, self.up_fmt, self.inter, self.hidden, self.n_expert)
+        self.down_fmt = conv(self.down, self.down_fmt, self.hidden, self.inter, self.n_expert)
+        if self.sh_inter:
+            self.sh_gate_fmt = conv(self.sh_gate, self.sh_gate_fmt, self.sh_inter, self.hidden, 1)
+            self.sh_up_fmt = conv(self.sh_up, self.sh_up_fmt, self.sh_inter, self.hidden, 1)
+            self.sh_down_fmt = conv(self.sh_down, self.sh_down_fmt, self.hidden, self.sh_inter, 1)
+        return self
 
 
 class MoeLayer:

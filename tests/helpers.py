@@ -95,8 +95,9 @@ def host_inputs(s: Shape, T: int, logit_shift: Optional[np.ndarray] = None):
     return x, logits, bias
 
 
-def device_weights(s: Shape, device="cuda", block=False):
-    """The same layer generated on the GPU (identical bytes)."""
+def device_weights(s: Shape, device="cuda", block=False, planar=False):
+    """The same layer generated on the GPU (identical bytes); planar: its MXFP4 tensors then
+    rewritten into the planar form."""
     import torch
     from deepstrix_amd.executor import LayerWeights
     gate = synth.weights_dev(s.gate_fmt, s.seed, synth.T_GATE, s.n_expert * s.inter, s.hidden)
@@ -119,6 +120,8 @@ def device_weights(s: Shape, device="cuda", block=False):
         w.norm_w = synth.normal_dev(s.seed, synth.T_NORM_W, s.hidden, 0.02, 1.0)
         w.router_w = synth.normal_dev(s.seed, synth.T_ROUTER_W, s.n_expert * s.hidden, 0.02)
         w.norm_eps = 1e-6
+    if planar:
+        w.to_planar()
     torch.cuda.synchronize()
     return w
 
