@@ -101,12 +101,13 @@ __device__ __forceinline__ void split_q4(uint32_t q, uint32_t &hi_word, uint32_t
 //   [half h][plane][block g][16 B]  (2 x 128 B)  then  [half h][plane][block g][8 B]  (2 x 64 B)
 // the first 16 and the last 8 bytes of the 24-byte operand of (plane, block 4 h + g); plane 0 =
 // high.  Rows are 128 bytes apart in multiples, so the 128-byte runs are whole cache lines.  The
-// n_sb block scales d follow the tiles.
+// n_sb block scales d follow the tiles, padded to a multiple of four (readers fetch them four at
+// a time).
 // ---------------------------------------------------------------------------------------
 constexpr uint32_t kStaged6Bytes = 384;
 constexpr int kScaleB6High = 134, kScaleB6Low = 130;
 __host__ __device__ inline uint32_t staged6_row_bytes(uint32_t n_sb) {
-    return (n_sb * (kStaged6Bytes + 4u) + 127u) & ~127u;
+    return (n_sb * kStaged6Bytes + ((n_sb + 3u) & ~3u) * 4u + 127u) & ~127u;
 }
 // Four int8 values (one per byte of `q`, any order) -> their codes of the high and of the low
 // plane, one per byte, same order.

@@ -40,12 +40,16 @@ constexpr int kGemmRF = 2;                  // 16-row fragments per wave and row
 constexpr int kGemmMT = 128;                // token columns per workgroup (the wide tile)
 constexpr int kGemmMTNarrow = 16;           // ... of the narrow tile: groups of a few members
 constexpr int kGemmAWaveBytes = 2 * kGemmRF * 2048 + 2 * 256;  // a wave's weights of one super-block
-// LDS of a workgroup with MT columns: two half super-blocks of the columns (each: 128 bytes per
-// column of operand heads, then 64 bytes per column of operand tails) | two rows of 128 block
-// scales (the loads that fill them are 64 lanes wide) | the waves' weight regions
-constexpr int gemm_half_bytes(int mt) { return mt * 192; }
-constexpr int gemm_yd_off(int mt) { return 2 * gemm_half_bytes(mt); }
-constexpr int gemm_a_off(int mt) { return gemm_yd_off(mt) + 2 * 128 * (int)sizeof(float); }
+// LDS of a workgroup with MT columns: the operand heads of two half super-blocks of the columns
+// (128 bytes per column each) | the operand tails of two super-blocks (128 bytes per column each:
+// both halves, one cache line) | two times 4 block scales of every column (the loads that fill them
+// are 64 lanes wide: 1 KB per 64 columns) | the waves' weight regions
+constexpr int gemm_heads_bytes(int mt) { return mt * 128; }
+constexpr int gemm_tails_off(int mt) { return 2 * gemm_heads_bytes(mt); }
+constexpr int gemm_tails_bytes(int mt) { return mt * 128; }
+constexpr int gemm_yd_off(int mt) { return gemm_tails_off(mt) + 2 * gemm_tails_bytes(mt); }
+constexpr int gemm_yd_bytes(int mt) { return mt > 64 ? 2048 : 1024; }
+constexpr int gemm_a_off(int mt) { return gemm_yd_off(mt) + 2 * gemm_yd_bytes(mt); }
 constexpr size_t gemm_lds_bytes(int mt) { return (size_t)gemm_a_off(mt) + kGemmWaves * kGemmAWaveBytes; }
 
 struct GemmParams {
@@ -80,8 +84,11 @@ __device__ __forceinline__ uint32_t gemm_dest_row(uint32_t m, uint32_t n_tokens,
 template <bool PAIR, int MT, bool PLANAR = false>
 __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp4_gemm(const GemmParams p) {
     constexpr int kGemmCG = MT / 16;                    // column groups
-    constexpr int kGemmHalfBytes = gemm_half_bytes(MT);  // half a super-block of all columns in LDS
+    constexpr int kHeadsBytes = gemm_heads_bytes(MT);    // the heads of half a super-block of all columns
+    constexpr int kTailsOff = gemm_tails_off(MT);
+    constexpr int kTailsBytes = gemm_tails_bytes(MT);    // the tails of a super-block of all columns
     constexpr int kGemmYdOff = gemm_yd_off(MT);
+    constexpr int kYdBytes = gemm_yd_bytes(MT);          // four block scales of all columns
     constexpr int kGemmAOff = gemm_a_off(MT);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ uint32_t s_dest[MT];
@@ -107,7 +114,9 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // Many column tiles per expert (skewed routing, many tokens): the items are dealt to the XCDs
     // like cards, which spreads the wide groups -- contiguous ranges of the list (it is by expert)
     // left the busiest XCD with 17 % more column groups than the average at Zipf-skewed routing,
-    // against 8 % (layer at T=4096: -4.6 %).  About a tile per expert: contiguous ranges, so that
+    // against 8 % (layer at T=4096: -4.6 %).  (One list per XCD that keeps every group's column
+    // tiles together, balanced to 1 % in items and column groups, fetches a quarter fewer bytes --
+    // neighbours share the weights in the XCD's L2 -- and is 6 % slower all the same.)  About a tile per expert: contiguous ranges, so that
     // an XCD streams one contiguous stretch of the weights (3-5 % faster then).
     const bool deal = n_items > p.n_expert + (p.n_expert >> 1);
     if (!deal && local >= (n_items + 7u) / 8u) return;  // uniform
@@ -215,9 +224,11 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // read side: lane (row n16, block g4) of fragment f: chunk g4 (first half), 4 + g4 (second)
     const uint32_t sw = ((n16 & 7u) * 8u + (g4 ^ (n16 & 7u))) * 16u;  // within a 1 KB slab
     const uint32_t a_rd = (n16 >> 3) * 1024u + sw;
-    // tails: column n16's 64 bytes hold chunk (2 plane + g4 / 2) at position chunk ^ (n16 / 4);
-    // the two planes' positions differ in one address bit
-    const uint32_t bt_rd = n16 * 64u + (((g4 >> 1) ^ (n16 >> 2)) * 16u) + (g4 & 1u) * 8u;
+    // tails: column n16's 128 bytes hold chunk (4 half + 2 plane + g4 / 2) at position
+    // chunk ^ (n16 % 8) ^ (n16 / 8): the even columns of a group take eight different positions and
+    // so do the odd ones, so that the 16 columns and their two 8-byte halves cover every bank once;
+    // half and plane each flip one address bit
+    const uint32_t bt_rd = n16 * 128u + (((g4 >> 1) ^ (n16 & 7u) ^ (n16 >> 3)) * 16u) + (g4 & 1u) * 8u;
     // sc: the lane's two scale bytes (block g4 of the first and of the second half), bytes 0 and 1
     struct GemmAFrag { uint4 a0, a1; uint32_t sc; };
     GemmAFrag a_cur[kGemmRF][2];
@@ -234,39 +245,44 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             }
     };
 
-    // B half h of super-block sb: of each column's 384 bytes the 128 at 128 h (the 16-byte heads of
-    // the operands of both planes and four blocks) and the 64 at 256 + 64 h (their 8-byte tails).
-    // The heads of the 8 columns 8 g .. 8 g + 7 are slab g of the half buffer's first part, fetched
-    // and swizzled like the weights; the tails of the wave's 16 columns are 1 KB of the second
-    // part: lane -> (column lane / 4, 16-byte chunk (lane % 4) ^ (column / 4)), so that 16 columns
-    // read at one chunk spread over all banks.
-    constexpr uint32_t kTailOff = (uint32_t)MT * 128u;   // of the tails inside a half buffer
+    // B of super-block sb: of each column's 384 bytes, per half h the 128 at 128 h (the 16-byte
+    // heads of the operands of both planes and four blocks), and once per super-block the 128 at
+    // 256 (their 8-byte tails, both halves: one cache line).  The heads of the 8 columns 8 g ..
+    // 8 g + 7 are slab g of a heads buffer, fetched and swizzled like the weights; the tails of the
+    // wave's 16 columns are two slabs of a tails buffer, fetched with the heads' lane offsets (the
+    // second slab's with one address bit flipped, see bt_rd).  The columns' block scales d come four
+    // super-blocks at a time (16 bytes per column, a wave per 64 columns).
     const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 2048u);
-    const uint32_t bt_lds = __builtin_amdgcn_readfirstlane(lds0 + kTailOff + wave * 1024u);
-    uint32_t b_fetch[2];  // column 16 w + 8 ii + l8, chunk c8 of the 128 bytes of heads
+    const uint32_t bt_lds = __builtin_amdgcn_readfirstlane(lds0 + kTailsOff + wave * 2048u);
+    uint32_t b_fetch[2];   // column 16 w + 8 ii + l8, chunk c8 = lane % 8 ^ l8 of a 128-byte run
 #pragma unroll
     for (int ii = 0; ii < 2; ii++)
         b_fetch[ii] = s_src[(wave * 16u + ii * 8u + l8) & (uint32_t)(MT - 1)] * p.act_row_bytes + c8 * 16u;
-    const uint32_t bt_fetch = s_src[(wave * 16u + (lane >> 2)) & (uint32_t)(MT - 1)] * p.act_row_bytes + 256u +
-                              (((lane & 3u) ^ ((lane >> 4) & 3u)) * 16u);
     const uint32_t yd_fetch = s_src[tid & (uint32_t)(MT - 1)] * p.act_row_bytes + p.n_sb * kStaged6Bytes;
-    const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 256u);
+    const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 1024u);
     // a wave whose 16 columns lie past the end of a short group fetches nothing (nobody reads
     // them: the column loop stops at the last group that holds a real column)
     const bool b_live = wave * 16u < cnt;
-    auto issue_b = [&](uint32_t sb, uint32_t h) {  // into half buffer h
+    auto issue_b = [&](uint32_t sb, uint32_t h) {  // the heads of half h, into heads buffer h
         if (!b_live) return;
         const uint8_t *src = p.act + (sb * kStaged6Bytes + h * 128u);
 #pragma unroll
         for (int ii = 0; ii < 2; ii++)
-            lds_dma16(b_lds + h * kGemmHalfBytes + (uint32_t)(ii * 1024), src, b_fetch[ii]);
-        lds_dma16(bt_lds + h * kGemmHalfBytes, p.act + (sb * kStaged6Bytes + h * 64u), bt_fetch);
+            lds_dma16(b_lds + h * kHeadsBytes + (uint32_t)(ii * 1024), src, b_fetch[ii]);
     };
-    auto issue_yd = [&](uint32_t sb) {  // waves 0 and 1: 64 columns each
-        if (wave < 2u) lds_dma4(yd_lds + (sb & 1u) * 512u, p.act + sb * 4u, yd_fetch);
+    auto issue_bt = [&](uint32_t sb) {  // the tails of both halves, into tails buffer sb % 2
+        if (!b_live) return;
+        const uint8_t *src = p.act + (sb * kStaged6Bytes + 256u);
+        lds_dma16(bt_lds + (sb & 1u) * kTailsBytes, src, b_fetch[0]);
+        lds_dma16(bt_lds + (sb & 1u) * kTailsBytes + 1024u, src, b_fetch[1] ^ 16u);
+    };
+    auto issue_yd = [&](uint32_t sb) {  // a wave per 64 columns: d of super-blocks sb .. sb + 3
+        if (wave < (uint32_t)(kYdBytes / 1024) && (sb & 3u) == 0u)
+            lds_dma16(yd_lds + ((sb >> 2) & 1u) * (uint32_t)kYdBytes, p.act + sb * 4u, yd_fetch);
     };
 
     issue_b(0, 0);
+    issue_bt(0);
     issue_yd(0);
 
     v4f acc[kGemmRF][2][kGemmCG];
@@ -295,13 +311,15 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     auto compute_half = [&](auto hc, auto njc, const uint32_t sb, const bool more) {
         constexpr int h = decltype(hc)::value;
         constexpr int NJ = decltype(njc)::value;
-        const uint8_t *half = tiles + h * kGemmHalfBytes;
-        const float *yds = s_yd + (sb & 1u) * 128u;
+        const uint8_t *half = tiles + h * kHeadsBytes;
+        const uint8_t *tails = tiles + kTailsOff + (sb & 1u) * kTailsBytes;
+        const float *yds = s_yd + ((sb >> 2) & 1u) * (uint32_t)(kYdBytes / 4) + (sb & 3u);
         // the operand of (column group j, plane q): 16 bytes of head, 8 of tail
         auto load_piece = [&](int j, int q) -> v8i {
             const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 1024u + sw) ^ ((uint32_t)q * 64u);
             const uint4 hd = *(const uint4 *)(half + cb);
-            const uint2 tl = *(const uint2 *)(half + kTailOff + (uint32_t)j * 1024u + (bt_rd ^ ((uint32_t)q * 32u)));
+            const uint2 tl = *(const uint2 *)(tails + (uint32_t)j * 2048u +
+                                              (bt_rd ^ ((uint32_t)q * 32u) ^ ((uint32_t)h * 64u)));
             return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
         };
         v4f c[kGemmRF][2];
@@ -314,7 +332,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
 #pragma unroll
         for (int pc = 0; pc < NP; pc++) {
             const int j = pc >> 1, q = pc & 1;
-            if (q == 0) yd = yds[j * 16u + n16];
+            if (q == 0) yd = yds[(j * 16u + n16) * 4u];
             if (pc + 1 < NP) ring[(pc + 1) & 1] = load_piece((pc + 1) >> 1, (pc + 1) & 1);
             DSX_PIN();
             v8i &bq = ring[pc & 1];
@@ -396,6 +414,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             __syncthreads();
             if (more) {
                 issue_b(sb + 1u, 0);
+                issue_bt(sb + 1u);
                 issue_yd(sb + 1u);
             }
             compute_half(std::integral_constant<int, 1>{}, njc, sb, more);
