@@ -122,6 +122,32 @@ def test_decode_modes_on_planar_weights(fused):
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32), err_msg=f"fused={fused} T={T}")
 
 
+def test_block_and_noalloc_entry_points_on_planar_weights():
+    """The residual block (norm, router matvec, layer, residual add) and the entry point without a
+    workspace run the same kernels on planar weights: bit for bit the row layout's results."""
+    import torch
+    from deepstrix_amd.executor import MoeLayer
+    s = SHAPES["all_mxfp4"]
+    rows = MoeLayer(H.device_weights(s, block=True), 130)
+    planar = MoeLayer(H.device_weights(s, block=True, planar=True), 130)
+    for T in (1, 3, 20, 130):
+        h, logits, _ = H.host_inputs(s, T)
+        a, b = torch.from_numpy(h.copy()).cuda(), torch.from_numpy(h.copy()).cuda()
+        rows.block(a)
+        planar.block(b)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), f"block T={T}"
+    for T in (1, 5):
+        x, logits, _ = H.host_inputs(s, T)
+        dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+        want = rows.run(dx, dl)
+        got = torch.full((T, s.hidden), float("nan"), dtype=torch.float32, device="cuda")
+        planar.run_noalloc(dx, dl, got)
+        torch.cuda.synchronize()
+        assert planar.status(builtin_scratch=True) == 0
+        assert torch.equal(want, got), f"noalloc T={T}"
+
+
 def test_a_layer_with_both_layouts_is_refused():
     from deepstrix_amd.executor import MoeLayer
     s = SHAPES["all_mxfp4"]
