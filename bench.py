@@ -176,7 +176,8 @@ def mixed_leg(H, torch, np, T=512):
     s = H.CFG5
     rng = np.random.default_rng(55)
     x, _, _ = H.host_inputs(s, T)
-    layer = MoeLayer(H.device_weights(s), T)
+    layers = {"": MoeLayer(H.device_weights(s), T),
+              "_planar_weights": MoeLayer(H.device_weights(s, planar=True), T)}   # (the MXFP4 gate/up matrices)
     dx = torch.from_numpy(x).cuda()
     dw = torch.from_numpy(rng.uniform(0.05, 0.6, (T, s.n_used)).astype(np.float32)).cuda()
     out = torch.empty((T, s.hidden), dtype=torch.float32, device="cuda")
@@ -186,16 +187,17 @@ def mixed_leg(H, torch, np, T=512):
     res = {"tokens": T}
     for name, sel in cases.items():
         ds = torch.from_numpy(sel).cuda()
-        for _ in range(2):
-            layer.run(dx, None, out=out, selected_in=ds, weights_in=dw)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        reps = 8
-        for _ in range(reps):
-            layer.run(dx, None, out=out, selected_in=ds, weights_in=dw)
-        torch.cuda.synchronize()
-        res[f"{name}_ms_per_layer"] = (time.perf_counter() - t0) / reps * 1e3
-    del layer
+        for tag, layer in layers.items():
+            for _ in range(2):
+                layer.run(dx, None, out=out, selected_in=ds, weights_in=dw)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            reps = 8
+            for _ in range(reps):
+                layer.run(dx, None, out=out, selected_in=ds, weights_in=dw)
+            torch.cuda.synchronize()
+            res[f"{name}_ms_per_layer{tag}"] = (time.perf_counter() - t0) / reps * 1e3
+    del layers, layer
     torch.cuda.empty_cache()
     return res
 
@@ -394,6 +396,21 @@ def main():
             lps[i % L].run(x_all[i:i + 1], lg_all[i:i + 1], out=out)
         torch.cuda.synchronize()
         extra["us_per_token_T1_planar_weights"] = (time.perf_counter() - t1) * 1e6 / K
+        # ... and the other token counts of config 2 (the grouped GEMMs from 40 tokens on)
+        for T in (() if (args.no_extra or args.no_small_t) else (4, 16, 64)):
+            xs, ls, _ = H.host_inputs(H.Shape(**{**base.__dict__, "seed": base.seed + T}), T)
+            xs, ls = torch.from_numpy(xs).cuda(), torch.from_numpy(ls).cuda()
+            o = torch.empty((T, base.hidden), dtype=torch.float32, device="cuda")
+            lpt = [MoeLayer(lp.w, T) for lp in lps]
+            for r in range(2):
+                lpt[r % L].run(xs, ls, out=o)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for r in range(8):
+                lpt[r % L].run(xs, ls, out=o)
+            torch.cuda.synchronize()
+            extra[f"us_per_token_T{T}_planar_weights"] = (time.perf_counter() - t1) * 1e6 / 8 / T
+            del lpt
         del lps
     if not args.no_chain:
         extra["chain_8_layers_T2"] = chain_leg(H, torch, np)

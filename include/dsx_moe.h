@@ -49,7 +49,7 @@ extern "C" {
  * -- each one whole cache line when the matrix is 128-byte aligned -- and then the 8-byte scale
  * groups as [super-block][row in tile].  Same size, same arithmetic, bit-identical results; the
  * grouped GEMMs of dsx_moe_layer_forward fetch such a matrix with about a third of the memory
- * requests (10 % faster at 4096 tokens).  Taken by dsx_moe_layer_create (every MXFP4 tensor of a
+ * requests (10 % faster at 4096 tokens, 25 % at 96 to 512, where they only stream weights).  Taken by dsx_moe_layer_create (every MXFP4 tensor of a
  * layer in the same form), dsx_dense_ffn and the four dsx_moe_* expert products. */
 #define DSX_FMT_MXFP4_PLANAR 1039
 
@@ -292,7 +292,7 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
                                      void *down_end);
 /* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens (default 100): from this many tokens on, a layer with MXFP4 gate/up runs the
+ * gemm_min_tokens (default 100; 40 on planar weights): from this many tokens on, a layer with MXFP4 gate/up runs the
  * grouped-GEMM path (128 token columns per work item, shared expert as an extra group; a Q8_0
  * down matrix takes the int8 grouped GEMM); an all-MXFP4 layer whose GEMMs use the narrow tile
  * (below) switches at 11/16 of it.

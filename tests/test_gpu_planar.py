@@ -95,6 +95,9 @@ def test_layer_is_bitwise_the_same_on_planar_weights(name):
     dwp = H.device_weights(s, planar=True)
     assert dwp.gate_fmt == FMT_MXFP4_PLANAR
     planar = MoeLayer(dwp, max(TOKENS))
+    # a planar layer takes the grouped GEMMs from 40 tokens on: the row layout follows it here, so
+    # that both run the same kernels at every token count
+    rows.set_tuning(gemm_min_tokens=40)
     hw = H.host_weights(s)
     for T in TOKENS:
         a, sel_a, w_a, x = _run(rows, s, T)
@@ -130,6 +133,7 @@ def test_block_and_noalloc_entry_points_on_planar_weights():
     s = SHAPES["all_mxfp4"]
     rows = MoeLayer(H.device_weights(s, block=True), 130)
     planar = MoeLayer(H.device_weights(s, block=True, planar=True), 130)
+    rows.set_tuning(gemm_min_tokens=40)
     for T in (1, 3, 20, 130):
         h, logits, _ = H.host_inputs(s, T)
         a, b = torch.from_numpy(h.copy()).cuda(), torch.from_numpy(h.copy()).cuda()
@@ -164,7 +168,8 @@ def test_v3_shape_planar_against_rows():
     s = H.CFG2
     rows = MoeLayer(H.device_weights(s), 600)
     planar = MoeLayer(H.device_weights(s, planar=True), 600)
-    for T in (1, 6, 33, 600):
+    rows.set_tuning(gemm_min_tokens=40)
+    for T in (1, 6, 33, 48, 600):
         a, _, _, _ = _run(rows, s, T)
         b, _, _, _ = _run(planar, s, T)
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32), err_msg=f"T={T}")
