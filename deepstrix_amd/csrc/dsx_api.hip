@@ -101,6 +101,8 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gemm<false, kGemmMTNarrow>);
         allow_lds(k_mxfp4_gemm<true, kGemmMT, true>);
         allow_lds(k_mxfp4_gemm<false, kGemmMT, true>);
+        allow_lds(k_mxfp4_gemm<true, kGemmMTNarrow, true>);
+        allow_lds(k_mxfp4_gemm<false, kGemmMTNarrow, true>);
         allow_lds(k_mxfp4_relayout<true>);
         allow_lds(k_mxfp4_relayout<false>);
         allow_lds(k_mxfp4_down_decode<false>);
@@ -178,7 +180,7 @@ int group_build_big(hipStream_t st, int32_t *group_count, int32_t *group_offset,
 
 // Grouped GEMM launch; max_wi bounds the number of work items, MT is the chunk they were built
 // with (kGemmMT or kGemmMTNarrow).
-// planar: the weights are in the planar form (wide tile only).
+// planar: the weights are in the planar form.
 template <bool PAIR, int MT = kGemmMT>
 int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi, bool planar = false) {
     if (max_wi == 0) return DSX_OK;
@@ -190,14 +192,10 @@ int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi, bool plana
     if ((uint64_t)p.n_rows * p.n_sb * kSuperBytes > 0xFFFFFFFFull ||
         act_rows * p.act_row_bytes > 0xFFFFFFFFull)
         return fail(DSX_ERR_INVALID_ARG, "gemm: a weight matrix or the activation rows exceed 4 GiB");
-    if constexpr (MT == kGemmMT) {
-        if (planar) {
-            hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT, true>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
-                               gemm_lds_bytes(MT), st, p);
-            return launched(PAIR ? "gate_up gemm" : "down gemm");
-        }
-    } else if (planar) {
-        return fail(DSX_ERR_UNSUPPORTED, "gemm: the narrow tile reads the engine's row layout only");
+    if (planar) {
+        hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT, true>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
+                           gemm_lds_bytes(MT), st, p);
+        return launched(PAIR ? "gate_up gemm" : "down gemm");
     }
     hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
                        gemm_lds_bytes(MT), st, p);

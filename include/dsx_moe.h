@@ -292,14 +292,14 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
                                      void *down_end);
 /* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens (default 100; 40 on planar weights): from this many tokens on, a layer with MXFP4 gate/up runs the
+ * gemm_min_tokens (default 100; 17 on planar weights): from this many tokens on, a layer with MXFP4 gate/up runs the
  * grouped-GEMM path (128 token columns per work item, shared expert as an extra group; a Q8_0
- * down matrix takes the int8 grouped GEMM); an all-MXFP4 layer whose GEMMs use the narrow tile
- * (below) switches at 11/16 of it.
- * decode_max_tokens (default 16): up to this many tokens, an all-MXFP4 layer runs the decode path
+ * down matrix takes the int8 grouped GEMM -- layers with a Q8_0 matrix keep 100 on planar weights too);
+ * an all-MXFP4 layer whose GEMMs use the narrow tile (below) switches at 11/16 of it.
+ * decode_max_tokens (default 16; 11 on planar weights): up to this many tokens, an all-MXFP4 layer runs the decode path
  * (dsx_moe_layer_set_decode: every token on its own picks, no grouping by expert; the one-launch
  * form serves at most 16 tokens, beyond that the decode kernels run once per stage).
- * gemm_narrow_members (default 1 = never): while the picks per expert average less than this,
+ * gemm_narrow_members (default 1 = never; 14 on planar weights): while the picks per expert average less than this,
  * the all-MXFP4 grouped GEMMs use 16 token columns per work item and two workgroups per CU. */
 int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
                              uint32_t decode_max_tokens, uint32_t gemm_narrow_members);

@@ -75,7 +75,8 @@ SHAPES = {
     "wide_shared": H.Shape(1024, 512, 16, 4, sh_inter=768, seed=45, **SMALL),
     "no_shared": H.Shape(1024, 512, 16, 4, shared=False, seed=46, **SMALL),
 }
-TOKENS = [1, 2, 3, 4, 7, 16, 17, 40, 99, 100, 130, 300]
+TOKENS = [1, 2, 3, 4, 7, 11, 12, 16, 17, 40, 99, 100, 130, 300]
+PLANAR_TUNING = dict(gemm_min_tokens=17, decode_max_tokens=11, gemm_narrow_members=14)
 
 
 def _run(layer, s, T):
@@ -95,16 +96,18 @@ def test_layer_is_bitwise_the_same_on_planar_weights(name):
     dwp = H.device_weights(s, planar=True)
     assert dwp.gate_fmt == FMT_MXFP4_PLANAR
     planar = MoeLayer(dwp, max(TOKENS))
-    # a planar layer takes the grouped GEMMs from 40 tokens on: the row layout follows it here, so
-    # that both run the same kernels at every token count
-    rows.set_tuning(gemm_min_tokens=40)
+    # a planar layer has its own thresholds (decode up to 11 tokens, then the grouped GEMMs, narrow
+    # tile first): the row layout follows them here, so that both run the same kernels at every
+    # token count
+    if s.down_fmt == FMT_MXFP4:   # (a layer with a Q8_0 matrix keeps the row layout's thresholds)
+        rows.set_tuning(**PLANAR_TUNING)
     hw = H.host_weights(s)
     for T in TOKENS:
         a, sel_a, w_a, x = _run(rows, s, T)
         b, sel_b, w_b, _ = _run(planar, s, T)
         np.testing.assert_array_equal(sel_a, sel_b)
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32), err_msg=f"{name} T={T}")
-        if T in (1, 4, 40, 130):
+        if T in (1, 4, 12, 40, 130):
             want = ref.moe_forward(hw, x, sel_b, w_b)
             H.assert_close(b, want, 2e-3, f"{name} planar T={T}")
 
@@ -119,6 +122,7 @@ def test_decode_modes_on_planar_weights(fused):
     planar = MoeLayer(H.device_weights(s, planar=True), 16)
     rows.set_decode(fused)
     planar.set_decode(fused)
+    planar.set_tuning(decode_max_tokens=16)   # (a planar layer leaves the decode path at 12 tokens)
     for T in (1, 2, 5, 12, 16):
         a, _, _, _ = _run(rows, s, T)
         b, _, _, _ = _run(planar, s, T)
@@ -133,7 +137,7 @@ def test_block_and_noalloc_entry_points_on_planar_weights():
     s = SHAPES["all_mxfp4"]
     rows = MoeLayer(H.device_weights(s, block=True), 130)
     planar = MoeLayer(H.device_weights(s, block=True, planar=True), 130)
-    rows.set_tuning(gemm_min_tokens=40)
+    rows.set_tuning(**PLANAR_TUNING)
     for T in (1, 3, 20, 130):
         h, logits, _ = H.host_inputs(s, T)
         a, b = torch.from_numpy(h.copy()).cuda(), torch.from_numpy(h.copy()).cuda()
@@ -168,7 +172,7 @@ def test_v3_shape_planar_against_rows():
     s = H.CFG2
     rows = MoeLayer(H.device_weights(s), 600)
     planar = MoeLayer(H.device_weights(s, planar=True), 600)
-    rows.set_tuning(gemm_min_tokens=40)
+    rows.set_tuning(**PLANAR_TUNING)
     for T in (1, 6, 33, 48, 600):
         a, _, _, _ = _run(rows, s, T)
         b, _, _, _ = _run(planar, s, T)
