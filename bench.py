@@ -30,7 +30,7 @@ COPY_BYTES = 256 << 20                    # size of the calibration copy (read 2
 
 # The dominant kernel of a decode step: one launch that streams gate, up and down of the 8
 # picks and the shared expert.
-DOMINANT_KERNEL = "k_mxfp4_decode_fused<8,false>"
+DOMINANT_KERNEL = "k_mxfp4_decode_fused<8,false,false>"
 # HBM bytes one launch of it moves come from hardware counters (two `rocprofv3 --pmc` runs of
 # this script: FETCH_SIZE, then WRITE_SIZE, each scaled by what it reads for the calibration
 # copy below, whose traffic is known).  The figure is read from the committed summary, which
