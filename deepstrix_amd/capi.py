@@ -84,6 +84,8 @@ SIGNATURES = {
     "dsx_dequant_rows": (_int, [_vp, _int, _vp, _vp, _u32, _u32]),
     "dsx_moe_layer_create": (_int, [C.POINTER(LayerDesc), C.POINTER(_vp)]),
     "dsx_moe_layer_destroy": (None, [_vp]),
+    "dsx_moe_layer_weights_to_planar": (_int, [_vp, _vp]),
+    "dsx_moe_layer_weights_to_rows": (_int, [_vp, _vp]),
     "dsx_moe_layer_set_profile_events": (_int, [_vp, _vp, _vp, _vp]),
     "dsx_moe_layer_set_tuning": (_int, [_vp, _u32, _u32, _u32, _u32]),
     "dsx_moe_layer_set_decode": (_int, [_vp, _u32, _u32]),

@@ -112,6 +112,22 @@ class MoeLayer:
             except Exception:  # interpreter shutdown: the module globals are already gone
                 pass
 
+    def weights_to_planar(self):
+        """Rewrites the layer's MXFP4 tensors (self.w's buffers) in place into the planar form and
+        switches the layer over (include/dsx_moe.h: dsx_moe_layer_weights_to_planar)."""
+        check(lib().dsx_moe_layer_weights_to_planar(self._h, torch.cuda.current_stream().cuda_stream))
+        w = self.w
+        for name in ("gate_fmt", "up_fmt", "down_fmt") + (("sh_gate_fmt", "sh_up_fmt", "sh_down_fmt") if w.sh_inter else ()):
+            if getattr(w, name) == FMT_MXFP4:
+                setattr(w, name, FMT_MXFP4_PLANAR)
+
+    def weights_to_rows(self):
+        check(lib().dsx_moe_layer_weights_to_rows(self._h, torch.cuda.current_stream().cuda_stream))
+        w = self.w
+        for name in ("gate_fmt", "up_fmt", "down_fmt") + (("sh_gate_fmt", "sh_up_fmt", "sh_down_fmt") if w.sh_inter else ()):
+            if getattr(w, name) == FMT_MXFP4_PLANAR:
+                setattr(w, name, FMT_MXFP4)
+
     def set_profile_events(self, gate_up_begin=None, gate_up_end=None, down_end=None):
         """hipEvent_t handles (ints) recorded around the gate/up launch and after down."""
         check(lib().dsx_moe_layer_set_profile_events(self._h, gate_up_begin, gate_up_end, down_end))

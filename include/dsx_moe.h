@@ -285,6 +285,16 @@ typedef struct dsx_moe_layer dsx_moe_layer;
 
 int dsx_moe_layer_create(const dsx_moe_layer_desc *desc, dsx_moe_layer **out);
 void dsx_moe_layer_destroy(dsx_moe_layer *layer);
+/* No counterpart in the reference: rewrites every MXFP4 tensor the layer was created with -- the
+ * caller's weight buffers -- in place into the planar form (DSX_FMT_MXFP4_PLANAR above), or back
+ * into the engine's rows, and switches the layer over (its default thresholds included: a planar
+ * layer leaves the decode path at 12 tokens and starts with the 16-column GEMM tile).  A layer
+ * without MXFP4 tensors, or one already in the form asked for, is left as it is.  Shapes are
+ * checked before the first byte moves.  Stream-ordered like a kernel launch; nothing else may use
+ * the buffers in the other form afterwards (two layers over the same buffers must both be
+ * switched, the second one by creating it with the new format ids). */
+int dsx_moe_layer_weights_to_planar(dsx_moe_layer *layer, dsx_stream_t stream);
+int dsx_moe_layer_weights_to_rows(dsx_moe_layer *layer, dsx_stream_t stream);
 /* Measurement aid with no counterpart in the reference: hipEvent_t handles (or NULL) that
  * dsx_moe_layer_forward records on its stream right before and right after the gate/up
  * launch and after the down launch, so a harness can time the dominant kernel in place. */

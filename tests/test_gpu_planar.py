@@ -156,6 +156,35 @@ def test_block_and_noalloc_entry_points_on_planar_weights():
         assert torch.equal(want, got), f"noalloc T={T}"
 
 
+@pytest.mark.parametrize("name", ["all_mxfp4", "q8_shared", "q8_down"])
+def test_a_layer_switches_its_own_weights_over_and_back(name):
+    """dsx_moe_layer_weights_to_planar on a layer made on the engine's rows: the buffers become
+    what the conversion entry point makes of them, the layer computes what a layer created on
+    planar weights computes, and the way back restores the bytes."""
+    import torch
+    from deepstrix_amd.executor import MoeLayer
+    s = SHAPES[name]
+    dw = H.device_weights(s)
+    before = dw.gate.clone()
+    layer = MoeLayer(dw, 130)
+    want_planar = H.device_weights(s, planar=True)
+    ref_layer = MoeLayer(want_planar, 130)
+    layer.weights_to_planar()
+    torch.cuda.synchronize()
+    assert torch.equal(dw.gate, want_planar.gate) and torch.equal(dw.down, want_planar.down)
+    assert dw.gate_fmt == want_planar.gate_fmt and dw.down_fmt == want_planar.down_fmt
+    for T in (1, 14, 60, 130):
+        a, _, _, _ = _run(layer, s, T)
+        b, _, _, _ = _run(ref_layer, s, T)
+        np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32), err_msg=f"{name} T={T}")
+    layer.weights_to_planar()   # a second call changes nothing
+    torch.cuda.synchronize()
+    assert torch.equal(dw.gate, want_planar.gate)
+    layer.weights_to_rows()
+    torch.cuda.synchronize()
+    assert torch.equal(dw.gate, before) and dw.gate_fmt == FMT_MXFP4
+
+
 def test_a_layer_with_both_layouts_is_refused():
     from deepstrix_amd.executor import MoeLayer
     s = SHAPES["all_mxfp4"]
