@@ -202,13 +202,13 @@ def mixed_leg(H, torch, np, T=512):
     return res
 
 
-def chain_leg(H, torch, np, n_layers=8, T=2, steps=256):
+def chain_leg(H, torch, np, n_layers=8, T=2, steps=256, planar=False):
     """BASELINE config 4: 8 chained V3-shape MXFP4 layers, each h += MoE(RMSNorm(h)), T = 2
     tokens per step, 256 consecutive steps with fresh N(0,1) inputs.  Latency of one step from
     the host's point of view (submit + run + synchronize), eager and replayed from a graph."""
     from deepstrix_amd.executor import MoeChain
     shapes = [H.Shape(**{**H.CFG2.__dict__, "seed": H.CFG2.seed + 0x1000 + 0x100 * i}) for i in range(n_layers)]
-    chain = MoeChain([H.device_weights(s, block=True) for s in shapes], T)
+    chain = MoeChain([H.device_weights(s, block=True, planar=planar) for s in shapes], T)
     hidden = H.CFG2.hidden
     inputs = torch.randn((steps, T, hidden), dtype=torch.float32, device="cuda",
                          generator=torch.Generator(device="cuda").manual_seed(4))
@@ -414,6 +414,10 @@ def main():
         del lps
     if not args.no_chain:
         extra["chain_8_layers_T2"] = chain_leg(H, torch, np)
+        torch.cuda.empty_cache()
+        on_planar = chain_leg(H, torch, np, planar=True)
+        extra["chain_8_layers_T2"]["planar_weights"] = {k: on_planar[k] for k in ("eager_us_per_step", "graph_us_per_step")}
+        torch.cuda.empty_cache()
     if not args.no_extra:
         extra["mixed_precision_T512_cfg5"] = mixed_leg(H, torch, np)
         extra["q8_0_cfg1"] = q8_0_leg(H, torch, np)
