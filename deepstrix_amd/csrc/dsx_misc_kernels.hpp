@@ -588,12 +588,17 @@ __global__ __launch_bounds__(kGbThreads) void k_group_build(
     __shared__ int s_count[DSX_MAX_EXPERTS_K];
     __shared__ int s_off[DSX_MAX_EXPERTS_K + 1];
     __shared__ int s_wi_off[DSX_MAX_EXPERTS_K + 1];
+    // the picks, kept in LDS for the scatter below, which walks them once per expert (from global
+    // memory every walk step waits for a load: 44 ns per pick)
+    constexpr uint32_t kGbPicksInLds = 2048;
+    __shared__ int s_sel[kGbPicksInLds];
     const uint32_t tid = threadIdx.x;
     const uint32_t total = b * n_used;
     for (uint32_t e = tid; e < n_expert; e += kGbThreads) s_count[e] = 0;
     __syncthreads();
     for (uint32_t i = tid; i < total; i += kGbThreads) {
         const int e = selected[i];
+        if (i < kGbPicksInLds) s_sel[i] = e;
         if (e >= 0 && (uint32_t)e < n_expert) atomicAdd(&s_count[e], 1);
     }
     __syncthreads();
@@ -637,7 +642,7 @@ __global__ __launch_bounds__(kGbThreads) void k_group_build(
         uint32_t pos = (uint32_t)s_off[e];
         for (uint32_t i0 = 0; i0 < total; i0 += 64u) {
             const uint32_t i = i0 + lane;
-            const bool hit = (i < total) && (selected[i] == (int)e);
+            const bool hit = (i < total) && ((i < kGbPicksInLds ? s_sel[i] : selected[i]) == (int)e);
             const uint64_t mask = __ballot(hit);
             if (hit) {
                 const uint32_t before = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
