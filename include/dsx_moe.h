@@ -290,7 +290,7 @@ void dsx_moe_layer_destroy(dsx_moe_layer *layer);
  * into the engine's rows, and switches the layer over (its default thresholds included: a planar
  * layer leaves the decode path at 12 tokens and starts with the 16-column GEMM tile).  A layer
  * without MXFP4 tensors, or one already in the form asked for, is left as it is.  Shapes are
- * checked before the first byte moves.  Stream-ordered like a kernel launch; nothing else may use
+ * checked before the first byte moves; two MXFP4 tensors at one address are refused.  Stream-ordered like a kernel launch; nothing else may use
  * the buffers in the other form afterwards (two layers over the same buffers must both be
  * switched, the second one by creating it with the new format ids). */
 int dsx_moe_layer_weights_to_planar(dsx_moe_layer *layer, dsx_stream_t stream);

@@ -185,6 +185,21 @@ def test_a_layer_switches_its_own_weights_over_and_back(name):
     assert torch.equal(dw.gate, before) and dw.gate_fmt == FMT_MXFP4
 
 
+def test_a_layer_whose_tensors_share_memory_is_not_converted():
+    """gate and up over the same bytes would be rewritten twice: refused before anything moves."""
+    import torch
+    from deepstrix_amd.executor import MoeLayer
+    s = SHAPES["all_mxfp4"]
+    dw = H.device_weights(s)
+    dw.up = dw.gate
+    before = dw.gate.clone()
+    layer = MoeLayer(dw, 4)
+    with pytest.raises(DsxError):
+        layer.weights_to_planar()
+    torch.cuda.synchronize()
+    assert torch.equal(dw.gate, before)
+
+
 def test_a_layer_with_both_layouts_is_refused():
     from deepstrix_amd.executor import MoeLayer
     s = SHAPES["all_mxfp4"]
