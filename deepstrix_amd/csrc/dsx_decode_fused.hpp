@@ -113,6 +113,20 @@ __device__ __forceinline__ void df_store_f32(float *p, float v) {
 __device__ __forceinline__ float df_load_f32(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// One word at an address that is the same for the whole wave and was written before the launch.
+// SCALAR: through the scalar cache -- a vector load issued by a workgroup that starts on a busy CU
+// returns behind everything the CU has in flight, and an item cannot request its weights before
+// it knows its expert.  The instantiations that pair tokens (four tokens and more by default)
+// read their pick and routing weight this way: 1-3 % off a step at the DeepSeek-V3 shape.  With
+// one or two tokens most items start on an idle CU, and the scalar round trip in front of the
+// first weight request costs 1-2 % instead, so the other instantiations keep the vector load.
+template <bool SCALAR>
+__device__ __forceinline__ uint32_t df_uniform_u32(const void *addr) {
+    if (!SCALAR) return *(const uint32_t *)addr;
+    uint32_t v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(addr) : "memory");
+    return v;
+}
 
 // ---- which tokens an item serves ---------------------------------------------------------------
 // With sharing on, the tokens that name one expert in a step (the shared expert: all tokens) are
@@ -152,7 +166,7 @@ __device__ __forceinline__ DfPair df_pair(const DecodeFusedParams &p, uint32_t t
         }
         return r;
     }
-    r.ew0 = p.ew[t * p.n_used + slot];
+    r.ew0 = __uint_as_float(df_uniform_u32<SHARE>(p.ew + t * p.n_used + slot));
     if (!SHARE) return r;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t n = p.n_tokens * p.n_used, mine = t * p.n_used, after = mine + p.n_used;
@@ -462,7 +476,7 @@ __device__ __forceinline__ void df_gate_up_item(const DecodeFusedParams &p, uint
     float clamp = p.clamp;
     int e = -1;
     if (slot < p.n_used) {
-        e = p.selected[t * p.n_used + slot];
+        e = (int)df_uniform_u32<SHARE>(p.selected + t * p.n_used + slot);
         if (e < 0 || (uint32_t)e >= p.n_expert) return;  // empty slot: its down items skip it too
         gate_e = p.gate + (uint64_t)e * p.gbpe;
         up_e = p.up + (uint64_t)e * p.ubpe;
@@ -604,7 +618,7 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
     const uint8_t *down_e = p.sh_down;
     int e = -1;
     if (slot < p.n_used) {
-        e = p.selected[t * p.n_used + slot];
+        e = (int)df_uniform_u32<SHARE>(p.selected + t * p.n_used + slot);
         if (e < 0 || (uint32_t)e >= p.n_expert) {
             // empty slot: contributes zeros (the sum must still wait for the others)
             if (last) df_combine(p, t, row0, 0.0f, slot);
