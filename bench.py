@@ -265,7 +265,7 @@ def main():
     import torch
     from deepstrix_amd import capi
     from deepstrix_amd.executor import MoeLayer
-    from tests import helpers as H
+    from deepstrix_amd import workloads as H
 
     torch.cuda.set_device(0)
     capi.init()
@@ -373,16 +373,18 @@ def main():
         extra[f"us_per_token_T{T}"] = (time.perf_counter() - t1) * 1e6 / reps / T
 
     if not args.no_prefill:
-        # on the engine's rows (the layout a checkpoint loads into) and on the planar form of the
-        # same matrices (rewritten in place once after loading; identical results): the planar
-        # figures are the leg's own, the other layout's time is quoted beside them
-        on_rows = prefill_leg(layers[0].w, base, H, torch, np)
+        # The figures of the leg are those of the engine's weight rows -- the layout a checkpoint
+        # loads into and the one the drop-in boundary fixes.  The planar form of the same matrices
+        # (opt-in, rewritten in place once after loading; identical results) is quoted beside them.
+        pre = prefill_leg(layers[0].w, base, H, torch, np)
+        pre["weights_layout"] = "engine rows (136-byte v2 super-blocks)"
         dwp = H.device_weights(H.Shape(**base.__dict__), planar=True)
-        pre = prefill_leg(dwp, base, H, torch, np)
-        pre["weights_layout"] = ("planar (DSX_FMT_MXFP4_PLANAR: nibble blocks and scales in separate planes, "
-                                 "made in place by dsx_mxfp4_rows_to_planar)")
-        pre["ms_per_layer_engine_rows"] = on_rows["ms_per_layer"]
-        pre["tokens_per_s_engine_rows"] = on_rows["tokens_per_s"]
+        on_planar = prefill_leg(dwp, base, H, torch, np)
+        pre["planar_weights"] = {
+            "weights_layout": "planar (DSX_FMT_MXFP4_PLANAR: nibble blocks and scales in separate planes, "
+                              "made in place by dsx_mxfp4_rows_to_planar)",
+            "ms_per_layer": on_planar["ms_per_layer"], "tokens_per_s": on_planar["tokens_per_s"],
+            "roofline": on_planar["roofline"]}
         extra["prefill_T4096"] = pre
         # the decode step on planar weights, rotating over as many layers as the headline figure
         del dwp

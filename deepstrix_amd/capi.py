@@ -91,6 +91,7 @@ SIGNATURES = {
     "dsx_moe_layer_set_decode": (_int, [_vp, _u32, _u32]),
     "dsx_moe_layer_set_trace": (_int, [_vp, _vp, _sz]),
     "dsx_moe_layer_status": (_int, [_vp, _vp, C.POINTER(C.c_uint32)]),
+    "dsx_moe_layer_status_ptr": (_int, [_vp, _vp, C.POINTER(_vp)]),
     "dsx_moe_layer_workspace_bytes": (_sz, [_vp, _u32]),
     "dsx_moe_block_forward": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
     "dsx_moe_block_forward_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),

@@ -48,6 +48,7 @@ namespace dsx {
 constexpr int kDfWaves = 4;            // waves per workgroup (both item kinds)
 constexpr uint32_t kDfDownRows = 64;   // output rows of a down item: 16 per wave
 constexpr uint32_t kDfSpinLimit = 1u << 16;   // rounds of about half a microsecond
+constexpr uint32_t kDfSpinLimitMax = 1u << 20;   // the most a caller may ask for (about half a second)
 constexpr uint32_t kDfFan = 32;        // copies of a slot's ready flag, one cache line each
 constexpr uint32_t kDfFanStride = 32;  // words between the copies (128 bytes)
 constexpr uint32_t kDfMaxTokens = 16;  // the flags are laid out for at most this many tokens
@@ -73,8 +74,7 @@ struct DecodeFusedParams {
     float *partials;                 // [n_tokens, n_slots, hidden]; kMidUnwritten on entry
     float *out;                      // [n_tokens, hidden]
     const float *residual;           // [n_tokens, hidden] or null; may alias out
-    const float *shared_rows;        // [n_tokens, hidden] or null: a shared expert computed elsewhere
-    uint32_t shared_async;           // ... by another stream, into rows marked unwritten: wait for them
+    const float *shared_rows;        // [n_tokens, hidden] or null: a shared expert computed before the launch
     uint32_t *slot_done;             // [n_tokens, n_slots], zero on entry
     uint32_t *ready;                 // [n_tokens, n_slots, kDfFan] flags kDfFanStride words apart, zero on entry
     uint32_t dn_early;               // super-blocks of a down item's weights requested before its mid row is checked
@@ -107,8 +107,15 @@ __device__ __forceinline__ uint32_t df_xcd_contiguous(uint32_t j, uint32_t n) {
     return (n & 7u) == 0u ? (j & 7u) * (n >> 3) + (j >> 3) : j;
 }
 
+// (A NaN is stored as the canonical quiet NaN: whatever bits an input or a weight produced, no
+// stored value can equal the unwritten pattern, itself a NaN, and make its readers wait.)
 __device__ __forceinline__ void df_store_f32(float *p, float v) {
+    v = v != v ? __uint_as_float(0x7FC00000u) : v;
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// What a reader makes of a value it gave up waiting for: zero.
+__device__ __forceinline__ float df_zero_if_unwritten(float v) {
+    return __float_as_uint(v) == kMidUnwritten ? 0.0f : v;
 }
 __device__ __forceinline__ float df_load_f32(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -547,7 +554,7 @@ __device__ __forceinline__ void df_relay_item(const DecodeFusedParams &p) {
 
 // ---- down item ---------------------------------------------------------------------------
 // Adds up the partial rows of token t for the wave's 16 rows [row0, row0 + 16): picks in slot
-// order, then the shared expert, then a shared expert computed elsewhere and the residual.  The
+// order, then the shared expert, then a shared expert computed before the launch and the residual.  The
 // caller is the item of the token's last slot in grid order, so the rows it reads come from
 // items that are running or done.  `own` (lane r < 16: row r) stands in for slot `own_slot`;
 // own_slot >= n_slots reads every slot from memory.
@@ -556,14 +563,9 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
     const uint32_t lane = threadIdx.x & 63u;
     const float *col = p.partials + (uint64_t)t * p.n_slots * p.hidden + row0 + (lane & 15u);
     float v[DSX_MAX_SLOTS];
-    float vs = 0.0f;   // the shared expert's value when another stream computes it
     const uint64_t o = (uint64_t)t * p.hidden + row0 + (lane & 15u);
     for (uint32_t spin = 0;; spin++) {
         bool missing = false;
-        if (p.shared_async && lane < 16u) {
-            vs = df_load_f32(p.shared_rows + o);
-            missing = __float_as_uint(vs) == kMidUnwritten;
-        }
 #pragma unroll
         for (int q = 0; q < DSX_MAX_SLOTS; q++) {
             v[q] = 0.0f;
@@ -575,6 +577,8 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
         if (__builtin_amdgcn_ballot_w64(missing) == 0ull) break;   // wave-uniform
         if (spin > p.spin_limit) {
             if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusPartialWaitExpired);
+#pragma unroll
+            for (int q = 0; q < DSX_MAX_SLOTS; q++) v[q] = df_zero_if_unwritten(v[q]);
             break;
         }
         __builtin_amdgcn_s_sleep(8);
@@ -584,7 +588,7 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
 #pragma unroll
         for (int q = 0; q < DSX_MAX_SLOTS; q++)
             if ((uint32_t)q < p.n_slots) s += (uint32_t)q == own_slot ? own : v[q];
-        if (p.shared_rows) s += p.shared_async ? vs : p.shared_rows[o];
+        if (p.shared_rows) s += p.shared_rows[o];
         if (p.residual) s += p.residual[o];
         p.out[o] = s;
     }
@@ -686,6 +690,10 @@ __device__ __forceinline__ void df_down_item(const DecodeFusedParams &p, uint32_
             for (uint32_t spin = 0; __builtin_amdgcn_ballot_w64(!landed(v)) != 0ull; spin++) {
                 if (spin > p.spin_limit) {
                     if (lane == 0) atomicCAS(p.status, kStatusOk, kStatusMidWaitExpired);
+                    v.x = df_zero_if_unwritten(v.x);
+                    v.y = df_zero_if_unwritten(v.y);
+                    v.z = df_zero_if_unwritten(v.z);
+                    v.w = df_zero_if_unwritten(v.w);
                     break;
                 }
                 if (!flag_seen) {

@@ -344,8 +344,9 @@ __global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up(const GateUpPar
         }
         const float v = swiglu_clamp(gs, us, clamp, s_ew[j]);
         float *dst = p.mid + (uint64_t)s_dest[j] * p.n_rows + row0 + rr;
-        if (FUSE_MIDQ)  // written through to memory: another XCD's workgroup will read it
-            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (FUSE_MIDQ)  // written through to memory: another XCD's workgroup will read it (a NaN as
+                        // the canonical one, so that no result equals the unwritten pattern)
+            __hip_atomic_store(dst, v != v ? __uint_as_float(0x7FC00000u) : v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
             *dst = v;
     }

@@ -835,6 +835,22 @@ __global__ __launch_bounds__(256) void k_vec_add_inplace(float *__restrict__ out
     if (i < n) out[i] += rhs[i];
 }
 
+// out = (a + b) + c  (c may be null; out may alias any of them): the routed experts' rows, a shared
+// expert computed beside them and the residual, in the order the reference adds them
+// (crates/v4flash-kernels/src/het/forward_prefill.rs:12227-12232).  n is a multiple of 4.
+__global__ __launch_bounds__(256) void k_add_rows(float *out, const float *a, const float *b,
+                                                  const float *c, uint64_t n4) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= n4) return;
+    const float4 va = ((const float4 *)a)[i], vb = ((const float4 *)b)[i];
+    float4 s = make_float4(va.x + vb.x, va.y + vb.y, va.z + vb.z, va.w + vb.w);
+    if (c) {
+        const float4 vc = ((const float4 *)c)[i];
+        s.x += vc.x; s.y += vc.y; s.z += vc.z; s.w += vc.w;
+    }
+    ((float4 *)out)[i] = s;
+}
+
 // crates/v4flash-kernels/kernels/swiglu_clamp_weighted.hip:16-37
 __global__ __launch_bounds__(256) void k_swiglu_clamp_weighted(float *__restrict__ mid,
                                                                const float *__restrict__ gate,

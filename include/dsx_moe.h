@@ -290,9 +290,15 @@ void dsx_moe_layer_destroy(dsx_moe_layer *layer);
  * into the engine's rows, and switches the layer over (its default thresholds included: a planar
  * layer leaves the decode path at 12 tokens and starts with the 16-column GEMM tile).  A layer
  * without MXFP4 tensors, or one already in the form asked for, is left as it is.  Shapes are
- * checked before the first byte moves; two MXFP4 tensors at one address are refused.  Stream-ordered like a kernel launch; nothing else may use
- * the buffers in the other form afterwards (two layers over the same buffers must both be
- * switched, the second one by creating it with the new format ids). */
+ * checked before the first byte moves; MXFP4 tensors whose byte ranges overlap are refused.
+ * The rewrite is enqueued on `stream` like a kernel launch, while the layer switches over on the
+ * host at once: a forward on ANOTHER stream must first be ordered behind `stream` (event or
+ * synchronization), or it reads tensors that are still being rewritten.  Thresholds the caller set
+ * with dsx_moe_layer_set_tuning are kept.  If the rewrite of one tensor fails, the ones already
+ * rewritten are turned back; should that fail too, the layer refuses every later forward
+ * (DSX_ERR_UNSUPPORTED).  Nothing else may use the buffers in the other form afterwards (two layers
+ * over the same buffers must both be switched, the second one by creating it with the new format
+ * ids). */
 int dsx_moe_layer_weights_to_planar(dsx_moe_layer *layer, dsx_stream_t stream);
 int dsx_moe_layer_weights_to_rows(dsx_moe_layer *layer, dsx_stream_t stream);
 /* Measurement aid with no counterpart in the reference: hipEvent_t handles (or NULL) that
@@ -323,7 +329,8 @@ int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uin
  * from 2 tokens on (for steps whose tokens mostly name the same experts, such as the
  * verification of consecutive draft tokens); 2 = one launch per stage; 0 keeps the current
  * value.  spin_limit (0 keeps): bound, in polling rounds of about half a microsecond, of every
- * wait one workgroup does for another. */
+ * wait one workgroup does for another; values above 2^20 are taken as 2^20, so that every wait
+ * stays bounded. */
 int dsx_moe_layer_set_decode(dsx_moe_layer *layer, uint32_t fused, uint32_t spin_limit);
 /* Measurement aid with no counterpart in the reference: a device buffer of n_items x 4 uint64
  * that the one-launch decode path fills with clock readings (constant 100 MHz counter) per
@@ -342,6 +349,10 @@ int dsx_moe_layer_set_trace(dsx_moe_layer *layer, uint64_t *trace, size_t n_item
 #define DSX_STATUS_MIDQ_WAIT_EXPIRED 2u /* the fused mid quantization gave up waiting for a tile */
 #define DSX_STATUS_PARTIAL_WAIT_EXPIRED 3u /* the slot-order sum gave up waiting for a partial row */
 int dsx_moe_layer_status(const dsx_moe_layer *layer, const void *workspace, uint32_t *host_out);
+/* The device address of that status word (no copy, no synchronization: safe under capture), for a
+ * caller that wants to test it on the device or copy it with a node of its own graph.  No
+ * counterpart in the reference. */
+int dsx_moe_layer_status_ptr(const dsx_moe_layer *layer, void *workspace, uint32_t **device_word);
 /* Bytes of caller-provided device scratch for up to max_tokens tokens. */
 size_t dsx_moe_layer_workspace_bytes(const dsx_moe_layer *layer, uint32_t max_tokens);
 /* out[t,:] = sum_slot expert(x[t]) + shared(x[t]);  x f32 [n_tokens, hidden],

@@ -47,7 +47,11 @@ def _compare(out_h, x, sel_h, w_h, hw, toks, what):
     return st
 
 
-def test_config3_T4096_zipf_prefill_against_the_oracle_on_chosen_tokens():
+@pytest.mark.parametrize("planar", [False, True], ids=["engine_rows", "planar"])
+def test_config3_T4096_zipf_prefill_against_the_oracle_on_chosen_tokens(planar):
+    """planar: the same layer after its MXFP4 tensors were rewritten into the planar form -- the
+    128-column GEMM instantiation for planar weights with the work items dealt to the XCDs (many
+    column tiles per expert), against the oracle and bitwise against the engine's rows."""
     s, T = H.CFG2, 4096
     shift = 0.416 * H.zipf_logit_shift(s.n_expert, 3)
     x, logits, bias = H.host_inputs(s, T, shift)
@@ -55,14 +59,24 @@ def test_config3_T4096_zipf_prefill_against_the_oracle_on_chosen_tokens():
     hw = H.host_weights_from_device(s, dw)
     layer = MoeLayer(dw, T)
     dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    what = "config 3 (planar weights)" if planar else "config 3"
+    if planar:
+        on_rows, sel_rows, w_rows = layer.run(dx, dl, want_routing=True)
+        layer.weights_to_planar()
+        torch.cuda.synchronize()
     out, sel, w = layer.run(dx, dl, want_routing=True)
     torch.cuda.synchronize()
+    if planar:
+        assert torch.equal(sel, sel_rows) and torch.equal(w, w_rows)
+        assert torch.equal(out, on_rows), "planar weights: output differs from the engine's rows"
     out_h, sel_h, w_h = out.cpu().numpy(), sel.cpu().numpy(), w.cpu().numpy()
     cnt = np.bincount(sel_h.ravel(), minlength=s.n_expert)
     assert cnt.max() > 16 * 128 and cnt.max() % 128 != 0          # many tiles, the last one ragged
+    # more work items than 1.5 x the experts: the kernel deals them to the XCDs
+    assert int(np.ceil(cnt / 128).sum()) + T // 128 > s.n_expert + s.n_expert // 2
     toks = _edge_tokens(sel_h, s.n_expert, 256)
     assert toks.size >= 256
-    _compare(out_h, x, sel_h, w_h, hw, toks, "config 3")
+    _compare(out_h, x, sel_h, w_h, hw, toks, what)
     # bit-stability: the same call again gives the same bits
     again = layer.run(dx, dl)
     assert torch.equal(again, out)
@@ -75,7 +89,7 @@ def test_config3_T4096_zipf_prefill_against_the_oracle_on_chosen_tokens():
     out2 = layer.run(dx, None, selected_in=torch.from_numpy(sel2).cuda(), weights_in=w)
     out2_h = out2.cpu().numpy()
     toks2 = np.unique(np.concatenate([np.arange(0, T, 3)[:96], np.arange(7, T, 97), toks[:64]]))
-    _compare(out2_h, x, sel2, w_h, hw, toks2, "config 3 with empty slots")
+    _compare(out2_h, x, sel2, w_h, hw, toks2, what + " with empty slots")
 
 
 def test_config5_T512_mixed_precision_against_the_oracle_on_chosen_tokens():

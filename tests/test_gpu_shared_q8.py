@@ -55,14 +55,16 @@ def test_small_layer_with_q8_0_shared_expert_of_another_width(T):
 
 
 def test_small_layer_pre_norm_block_with_q8_0_shared_expert():
-    """h += layer(RMSNorm(h)) with the residual folded into the one-launch decode path."""
+    """h += layer(RMSNorm(h)) with the residual folded into the one-launch decode path (up to three
+    tokens: the shared expert inside the launch; more: on the side stream, its rows and the
+    residual added behind the join while the launch writes to a row buffer of the workspace)."""
     s = SMALL
     dw = H.device_weights(s, block=True)
-    layer = MoeLayer(dw, 4)
+    layer = MoeLayer(dw, 8)
     norm_w, router_w = H.host_block_params(s)
     hw = H.host_weights(s)
     rng = np.random.default_rng(3)
-    for T in (1, 3):
+    for T in (1, 3, 5, 8):
         h0 = rng.standard_normal((T, s.hidden)).astype(np.float32)
         xn = ref.rms_norm(h0, norm_w, 1e-6)
         logits = ref.router_logits(router_w, xn)
