@@ -22,10 +22,11 @@
 // bytes per product halve against 64 columns) and loads in memory order (see below).
 //
 // The Q8_K block scale d of the activations differs per (column, super-block), so the
-// matrix pipe cannot carry a sum across super-blocks: each fragment's instructions of one
-// half super-block accumulate into a fresh register quad that is then folded into the
-// accumulator with the column's d (one FMA per value, on the vector ALU while the matrix
-// pipe runs the next fragment).
+// matrix pipe cannot carry a sum across super-blocks.  The wide tile runs a column group's four
+// operands of a super-block (half x plane) back to back through one register quad per weight
+// fragment and folds it into the accumulator with the column's d once per super-block (one FMA
+// per value, placed between the next column group's first matrix instructions); the narrow
+// tile, whose operands arrive by half super-blocks, folds once per half.
 #pragma once
 
 #include <type_traits>
@@ -40,17 +41,34 @@ constexpr int kGemmRF = 2;                  // 16-row fragments per wave and row
 constexpr int kGemmMT = 128;                // token columns per workgroup (the wide tile)
 constexpr int kGemmMTNarrow = 16;           // ... of the narrow tile: groups of a few members
 constexpr int kGemmAWaveBytes = 2 * kGemmRF * 2048 + 2 * 256;  // a wave's weights of one super-block
-// LDS of a workgroup with MT columns: the operand heads of two half super-blocks of the columns
-// (128 bytes per column each) | the operand tails of two super-blocks (128 bytes per column each:
-// both halves, one cache line) | two times 4 block scales of every column (the loads that fill them
-// are 64 lanes wide: 1 KB per 64 columns) | the waves' weight regions
+// LDS of a workgroup.
+// Narrow tile (MT = 16): the operand heads of two half super-blocks of the columns (128 bytes per
+// column each) | the operand tails of two super-blocks (128 bytes per column each: both halves,
+// one cache line) | two times 4 block scales of every column (the loads that fill them are 64
+// lanes wide: 1 KB per 64 columns) | the waves' weight regions.
+// Wide tile (MT = 128): two buffers of 64 columns x one whole super-block (384 bytes per column:
+// the heads of half 0, the heads of half 1, the tails; 8 KB each) | the block scales | the waves'
+// weight regions.
+constexpr int kGemmPhaseCols = 64;                       // columns of one buffer of the wide tile
+constexpr int kGemmPhaseLine = kGemmPhaseCols * 128;     // one of its three 128-byte lines per column
+constexpr int kGemmPhaseBytes = 3 * kGemmPhaseLine;
 constexpr int gemm_heads_bytes(int mt) { return mt * 128; }
 constexpr int gemm_tails_off(int mt) { return 2 * gemm_heads_bytes(mt); }
 constexpr int gemm_tails_bytes(int mt) { return mt * 128; }
-constexpr int gemm_yd_off(int mt) { return gemm_tails_off(mt) + 2 * gemm_tails_bytes(mt); }
+constexpr int gemm_yd_off(int mt) { return mt == kGemmMT ? 2 * kGemmPhaseBytes : gemm_tails_off(mt) + 2 * gemm_tails_bytes(mt); }
 constexpr int gemm_yd_bytes(int mt) { return mt > 64 ? 2048 : 1024; }
 constexpr int gemm_a_off(int mt) { return gemm_yd_off(mt) + 2 * gemm_yd_bytes(mt); }
 constexpr size_t gemm_lds_bytes(int mt) { return (size_t)gemm_a_off(mt) + kGemmWaves * kGemmAWaveBytes; }
+
+// f(integral_constant<int, I>) for I = From .. To - 1, unrolled at compile time (the matrix
+// instruction wants its format and scale-select arguments as constants)
+template <int From, int To, typename F>
+__device__ __forceinline__ void gemm_static_for(F &&f) {
+    if constexpr (From < To) {
+        f(std::integral_constant<int, From>{});
+        gemm_static_for<From + 1, To>(f);
+    }
+}
 
 struct GemmParams {
     const uint8_t *w0, *w1;        // [n_expert] experts (gate, up), or down in w0 (w1 unused)
@@ -210,7 +228,7 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // super-block, shared, double buffered; wave w fetches columns 16 w .. 16 w + 15.
     constexpr int kALoads = 4 * kGemmRF + 2;  // per wave and super-block
     // load L of those: 0..7 the halves of the four fragments, 8 and 9 the scales of the row sets
-    auto issue_a_one = [&](int L, uint32_t sb) {
+    auto issue_a_one = [&](int L, uint32_t sb) __attribute__((always_inline)) {
         if (L < 4 * kGemmRF) {
             const int f = L >> 1, i = L & 1, r = f >> 1, m = f & 1;
             lds_dma16(a_lds + (uint32_t)(f * 2048 + i * 1024),
@@ -252,192 +270,408 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // wave's 16 columns are two slabs of a tails buffer, fetched with the heads' lane offsets (the
     // second slab's with one address bit flipped, see bt_rd).  The columns' block scales d come four
     // super-blocks at a time (16 bytes per column, a wave per 64 columns).
-    const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 2048u);
-    const uint32_t bt_lds = __builtin_amdgcn_readfirstlane(lds0 + kTailsOff + wave * 2048u);
-    uint32_t b_fetch[2];   // column 16 w + 8 ii + l8, chunk c8 = lane % 8 ^ l8 of a 128-byte run
-#pragma unroll
-    for (int ii = 0; ii < 2; ii++)
-        b_fetch[ii] = s_src[(wave * 16u + ii * 8u + l8) & (uint32_t)(MT - 1)] * p.act_row_bytes + c8 * 16u;
     const uint32_t yd_fetch = s_src[tid & (uint32_t)(MT - 1)] * p.act_row_bytes + p.n_sb * kStaged6Bytes;
     const uint32_t yd_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmYdOff + (wave & 1u) * 1024u);
-    // a wave whose 16 columns lie past the end of a short group fetches nothing (nobody reads
-    // them: the column loop stops at the last group that holds a real column)
-    const bool b_live = wave * 16u < cnt;
-    auto issue_b = [&](uint32_t sb, uint32_t h) {  // the heads of half h, into heads buffer h
-        if (!b_live) return;
-        const uint8_t *src = p.act + (sb * kStaged6Bytes + h * 128u);
-#pragma unroll
-        for (int ii = 0; ii < 2; ii++)
-            lds_dma16(b_lds + h * kHeadsBytes + (uint32_t)(ii * 1024), src, b_fetch[ii]);
-    };
-    auto issue_bt = [&](uint32_t sb) {  // the tails of both halves, into tails buffer sb % 2
-        if (!b_live) return;
-        const uint8_t *src = p.act + (sb * kStaged6Bytes + 256u);
-        lds_dma16(bt_lds + (sb & 1u) * kTailsBytes, src, b_fetch[0]);
-        lds_dma16(bt_lds + (sb & 1u) * kTailsBytes + 1024u, src, b_fetch[1] ^ 16u);
-    };
     auto issue_yd = [&](uint32_t sb) {  // a wave per 64 columns: d of super-blocks sb .. sb + 3
         if (wave < (uint32_t)(kYdBytes / 1024) && (sb & 3u) == 0u)
             lds_dma16(yd_lds + ((sb >> 2) & 1u) * (uint32_t)kYdBytes, p.act + sb * 4u, yd_fetch);
     };
 
-    issue_b(0, 0);
-    issue_bt(0);
-    issue_yd(0);
-
     v4f acc[kGemmRF][2][kGemmCG];
+    if constexpr (MT == kGemmMT) {
+        // ---- the wide tile -------------------------------------------------------------------
+        // B comes in phases of 64 columns x one whole super-block (each column's three cache lines:
+        // heads of half 0, heads of half 1, tails), into two buffers that alternate.  A tile of
+        // more than 64 columns runs two phases per super-block (columns 0..63, then 64..127), a
+        // narrower one a single phase.  The loads of a phase go out at the start of the phase
+        // before it.  Inside a phase a column group's four operands (half x plane) are multiplied
+        // back to back against the wave's four weight fragments, so that the matrix pipe carries
+        // the sum over the whole super-block -- the reference's order, sum the eight blocks, then
+        // scale by the activations' d (crates/v4flash-kernels/src/mxfp4_tables.rs:52-73) -- and the
+        // vector ALU folds one quad per fragment and super-block.
+        const uint32_t bp_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024u);  // the wave's 8 columns: slab `wave`
+        uint32_t bp_fetch[2];   // column 64 ch + 8 w + l8, chunk c8 of a 128-byte line
 #pragma unroll
-    for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-        for (int m = 0; m < 2; m++)
-#pragma unroll
-            for (int j = 0; j < kGemmCG; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-
-    const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
-    // One half super-block with NJ column groups (compile-time, so the code below is one
-    // straight line): for every group, the two pieces (high and low plane) against the wave's
-    // four fragments, then the fold acc += d * c -- placed right before each fragment's
-    // temporary is overwritten by the next group's first piece.  The next piece's B operand is
-    // requested from LDS one piece ahead of its use (deeper changes nothing).  Empty asm
-    // statements pin that order; they emit no instruction, so the compiler still sees every
-    // real one and keeps its hazards.  Left alone it hoists every LDS read of the half to its
-    // top, which overflows the registers, pulls each fold up to the instruction that produces
-    // its input, where it waits, and with the group count as a run-time condition waits for
-    // each operand right after requesting it (layer at T=4096: 4.5 -> 4.0 ms).
-#define DSX_PIN() asm volatile("" ::: "memory")
-    auto compute_half = [&](auto hc, auto njc, const uint32_t sb, const bool more) {
-        constexpr int h = decltype(hc)::value;
-        constexpr int NJ = decltype(njc)::value;
-        const uint8_t *half = tiles + h * kHeadsBytes;
-        const uint8_t *tails = tiles + kTailsOff + (sb & 1u) * kTailsBytes;
-        const float *yds = s_yd + ((sb >> 2) & 1u) * (uint32_t)(kYdBytes / 4) + (sb & 3u);
-        // the operand of (column group j, plane q): 16 bytes of head, 8 of tail
-        auto load_piece = [&](int j, int q) -> v8i {
-            const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 1024u + sw) ^ ((uint32_t)q * 64u);
-            const uint4 hd = *(const uint4 *)(half + cb);
-            const uint2 tl = *(const uint2 *)(tails + (uint32_t)j * 2048u +
-                                              (bt_rd ^ ((uint32_t)q * 32u) ^ ((uint32_t)h * 64u)));
-            return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
+        for (int ch = 0; ch < 2; ch++)
+            bp_fetch[ch] = s_src[(uint32_t)ch * kGemmPhaseCols + wave * 8u + l8] * p.act_row_bytes + c8 * 16u;
+        // the second slab of a column group keeps its tails with one address bit flipped (bt_rd)
+        const uint32_t tflip = (wave & 1u) << 4;
+        // a wave whose column group lies past the end of a short group fetches nothing
+        const bool ph_live[2] = {(wave >> 1) * 16u < cnt, kGemmPhaseCols + (wave >> 1) * 16u < cnt};
+        auto issue_phase = [&](uint32_t sb, int ch, uint32_t buf) __attribute__((always_inline)) {
+            if (!ph_live[ch]) return;
+            // (uniform values, said so to the compiler: the loads take them in scalar registers)
+            const uint8_t *src = p.act + __builtin_amdgcn_readfirstlane(sb * kStaged6Bytes);
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(bp_lds + buf * (uint32_t)kGemmPhaseBytes);
+            lds_dma16(dst, src, bp_fetch[ch]);
+            lds_dma16(dst + (uint32_t)kGemmPhaseLine, src + 128, bp_fetch[ch]);
+            lds_dma16(dst + 2u * (uint32_t)kGemmPhaseLine, src + 256, bp_fetch[ch] ^ tflip);
         };
-        v4f c[kGemmRF][2];
-        // piece p = 2 j + q alternates between two operand registers
-        constexpr int NP = 2 * NJ;
-        v8i ring[2];
-        ring[0] = load_piece(0, 0);
-        float yd_prev = 0.0f, yd = 0.0f;
-        DSX_PIN();
+        issue_phase(0, 0, 0);
+        issue_yd(0);
+    #pragma unroll
+        for (int r = 0; r < kGemmRF; r++)
+    #pragma unroll
+            for (int m = 0; m < 2; m++)
+    #pragma unroll
+                for (int j = 0; j < kGemmCG; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+
+        // read side of a phase buffer: lane (column n16, block g4) of column group jj
+        uint32_t head_rd[2], tail_rd[2][2];
 #pragma unroll
-        for (int pc = 0; pc < NP; pc++) {
-            const int j = pc >> 1, q = pc & 1;
-            if (q == 0) yd = yds[(j * 16u + n16) * 4u];
-            if (pc + 1 < NP) ring[(pc + 1) & 1] = load_piece((pc + 1) >> 1, (pc + 1) & 1);
-            DSX_PIN();
-            v8i &bq = ring[pc & 1];
-            asm volatile("" : "+v"(bq));  // the products with this piece stay behind the request above
+        for (int q = 0; q < 2; q++) {
+            head_rd[q] = ((n16 >> 3) * 1024u + sw) ^ ((uint32_t)q * 64u);
+#pragma unroll
+            for (int h = 0; h < 2; h++) tail_rd[h][q] = 2u * (uint32_t)kGemmPhaseLine + (bt_rd ^ ((uint32_t)q * 32u) ^ ((uint32_t)h * 64u));
+        }
+        const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
+
+        // One phase: NJP column groups, the first of them column group J0 of the tile.  ALoads
+        // of the next super-block's weight loads, starting with load AFrom, go out one behind each
+        // of the first operands' products.
+        auto compute_phase = [&](auto njpc, auto j0c, auto afc, auto alc, const uint32_t buf, const uint32_t sb)
+                                 __attribute__((always_inline)) {
+            constexpr int NJP = decltype(njpc)::value, J0 = decltype(j0c)::value;
+            constexpr int AFrom = decltype(afc)::value, ALoads = decltype(alc)::value;
+            constexpr int NP = 4 * NJP;
+            const uint8_t *pb = tiles + buf * (uint32_t)kGemmPhaseBytes;
+            const float *yds = s_yd + ((sb >> 2) & 1u) * (uint32_t)(kYdBytes / 4) + (sb & 3u);
+            auto load_piece = [&](int jj, int pp) __attribute__((always_inline)) -> v8i {   // pp = 2 half + plane
+                const int h = pp >> 1, q = pp & 1;
+                const uint4 hd = *(const uint4 *)(pb + (uint32_t)(h * kGemmPhaseLine + jj * 2048) + head_rd[q]);
+                const uint2 tl = *(const uint2 *)(pb + (uint32_t)(jj * 2048) + tail_rd[h][q]);
+                return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
+            };
+            v4f c[kGemmRF][2];
+            v8i ring[2];
+            ring[0] = load_piece(0, 0);
+            float yd_prev = 0.0f, yd = 0.0f;
+            gemm_static_for<0, NP>([&](auto gpc) __attribute__((always_inline)) {
+                constexpr int gp = decltype(gpc)::value;
+                constexpr int jj = gp >> 2, pp = gp & 3, h = pp >> 1, q = pp & 1;
+                if (pp == 0) yd = yds[((uint32_t)(J0 + jj) * 16u + n16) * 4u];
+                if (gp + 1 < NP) ring[(gp + 1) & 1] = load_piece((gp + 1) >> 2, (gp + 1) & 3);
+                const v8i bq = ring[gp & 1];
+#pragma unroll
+                for (int r = 0; r < kGemmRF; r++)
+#pragma unroll
+                    for (int m = 0; m < 2; m++) {
+                        const GemmAFrag &w = a_cur[r][m];
+                        const uint4 &aw = h == 0 ? w.a0 : w.a1;
+                        const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
+                        if (pp == 0) {
+                            if (jj > 0) {   // the column group before: its sums are complete
+                                v4f &a = acc[r][m][J0 + (jj > 0 ? jj - 1 : 0)];
+                                a.x = fmaf(yd_prev, c[r][m].x, a.x);
+                                a.y = fmaf(yd_prev, c[r][m].y, a.y);
+                                a.z = fmaf(yd_prev, c[r][m].z, a.z);
+                                a.w = fmaf(yd_prev, c[r][m].w, a.w);
+                                // (the sums stay where they are written: without a use here the
+                                // compiler moves the products behind the next barrier, all operands live)
+                                asm volatile("" : "+v"(a));
+                            }
+                            c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 2, 0, (int)w.sc, 0, kScaleB6High);
+                        } else {
+                            c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                av, bq, c[r][m], 4, 2, h, (int)w.sc, 0, q == 0 ? kScaleB6High : kScaleB6Low);
+                        }
+                    }
+                if (pp == 3) yd_prev = yd;
+                if constexpr (gp < ALoads) {
+                    // literal indices: the load's registers are picked at compile time
+                    constexpr int kA = AFrom;
+                    if (gp == 0) issue_a_one(kA + 0 < kALoads ? kA + 0 : 0, sb + 1u);
+                    if (gp == 1) issue_a_one(kA + 1 < kALoads ? kA + 1 : 0, sb + 1u);
+                    if (gp == 2) issue_a_one(kA + 2 < kALoads ? kA + 2 : 0, sb + 1u);
+                    if (gp == 3) issue_a_one(kA + 3 < kALoads ? kA + 3 : 0, sb + 1u);
+                    if (gp == 4) issue_a_one(kA + 4 < kALoads ? kA + 4 : 0, sb + 1u);
+                    if (gp == 5) issue_a_one(kA + 5 < kALoads ? kA + 5 : 0, sb + 1u);
+                    if (gp == 6) issue_a_one(kA + 6 < kALoads ? kA + 6 : 0, sb + 1u);
+                    if (gp == 7) issue_a_one(kA + 7 < kALoads ? kA + 7 : 0, sb + 1u);
+                    if (gp == 8) issue_a_one(kA + 8 < kALoads ? kA + 8 : 0, sb + 1u);
+                    if (gp == 9) issue_a_one(kA + 9 < kALoads ? kA + 9 : 0, sb + 1u);
+                }
+                // Nothing moves across the end of an operand's products: the request of the next
+                // operand stays right ahead of them, the folds beside them.  (The empty statement
+                // orders the LDS reads, which the compiler otherwise hoists to the top of the loop
+                // -- more live operands than there are registers; the barrier holds the scheduler.)
+                asm volatile("" ::: "memory");
+                if constexpr (pp == 0 && jj > 0) {
+                    // a fragment's fold, then its first product: the matrix pipe starts on the new
+                    // column group after 4 vector instructions instead of 16
+#pragma unroll
+                    for (int f = 0; f < 2 * kGemmRF; f++) {
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // 4 x vector ALU
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 x matrix
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
 #pragma unroll
             for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
                 for (int m = 0; m < 2; m++) {
-                    const GemmAFrag &w = a_cur[r][m];
-                    const uint4 &aw = h == 0 ? w.a0 : w.a1;
-                    const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
-                    if (q == 0) {
-                        if (j > 0) {
-                            asm volatile("" : "+v"(c[r][m]));
-                            v4f &a = acc[r][m][j > 0 ? j - 1 : 0];
-                            a.x = fmaf(yd_prev, c[r][m].x, a.x);
-                            a.y = fmaf(yd_prev, c[r][m].y, a.y);
-                            a.z = fmaf(yd_prev, c[r][m].z, a.z);
-                            a.w = fmaf(yd_prev, c[r][m].w, a.w);
-                            asm volatile("" : "+v"(a));
-                        }
-                        c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                            av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 2, h, (int)w.sc, 0, kScaleB6High);
-                    } else {
-                        c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                            av, bq, c[r][m], 4, 2, h, (int)w.sc, 0, kScaleB6Low);
-                    }
+                    v4f &a = acc[r][m][J0 + NJP - 1];
+                    a.x = fmaf(yd_prev, c[r][m].x, a.x);
+                    a.y = fmaf(yd_prev, c[r][m].y, a.y);
+                    a.z = fmaf(yd_prev, c[r][m].z, a.z);
+                    a.w = fmaf(yd_prev, c[r][m].w, a.w);
+                    asm volatile("" : "+v"(a));
                 }
-            if (q == 1) yd_prev = yd;
-            // the next super-block's weights, a load or two behind each piece's products: a
-            // request that has to wait for room in the memory pipeline then holds back nothing
-            // that the matrix pipe does not already have
-            {
-                constexpr int kFrom = h == 0 ? 0 : kAFirst, kCnt = h == 0 ? kAFirst : kALoads - kAFirst;
-                // behind the first pieces of a half: 8 of the 10 in the first half, one per piece (a
-                // few per cent faster than 6 + 4 and than all 10 at once, measured at 4096 tokens)
-                constexpr int kSpan = h == 0 ? (NP < 8 ? NP : 8) : (NP + 1) / 2;
-                const int lo = pc * kCnt / kSpan, hi = (pc + 1) * kCnt / kSpan;
-                if (pc < kSpan && more) {
-                    // literal indices: the load's registers are picked at compile time
-                    if (0 < kCnt && lo <= 0 && 0 < hi) issue_a_one(kFrom + 0, sb + 1u);
-                    if (1 < kCnt && lo <= 1 && 1 < hi) issue_a_one(kFrom + 1, sb + 1u);
-                    if (2 < kCnt && lo <= 2 && 2 < hi) issue_a_one(kFrom + 2, sb + 1u);
-                    if (3 < kCnt && lo <= 3 && 3 < hi) issue_a_one(kFrom + 3, sb + 1u);
-                    if (4 < kCnt && lo <= 4 && 4 < hi) issue_a_one(kFrom + 4, sb + 1u);
-                    if (5 < kCnt && lo <= 5 && 5 < hi) issue_a_one(kFrom + 5, sb + 1u);
-                    if (6 < kCnt && lo <= 6 && 6 < hi) issue_a_one(kFrom + 6, sb + 1u);
-                    if (7 < kCnt && lo <= 7 && 7 < hi) issue_a_one(kFrom + 7, sb + 1u);
-                    if (8 < kCnt && lo <= 8 && 8 < hi) issue_a_one(kFrom + 8, sb + 1u);
-                    if (9 < kCnt && lo <= 9 && 9 < hi) issue_a_one(kFrom + 9, sb + 1u);
-                }
-            }
-        }
-        // fold the last group
-#pragma unroll
-        for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-            for (int m = 0; m < 2; m++) {
-                v4f &a = acc[r][m][NJ - 1];
-                a.x = fmaf(yd_prev, c[r][m].x, a.x);
-                a.y = fmaf(yd_prev, c[r][m].y, a.y);
-                a.z = fmaf(yd_prev, c[r][m].z, a.z);
-                a.w = fmaf(yd_prev, c[r][m].w, a.w);
-            }
-    };
-#undef DSX_PIN
-
-    auto main_loop = [&](auto njc) {
-        for (uint32_t sb = 0; sb < p.n_sb; sb++) {
-            const bool more = sb + 1u < p.n_sb;
+        };
+        using I0 = std::integral_constant<int, 0>;
+        // up to 64 columns: one phase per super-block, the buffers alternate by super-block
+        // (The last super-block, which requests nothing, is a copy of the loop body: a condition
+        // inside the body would split it into basic blocks, and the compiler then moves every
+        // matrix instruction into the last of them.)
+        using I1 = std::integral_constant<int, 1>;
+        auto step_one_phase = [&](auto njc, auto morec, const uint32_t sb) __attribute__((always_inline)) {
+            constexpr int NJ = decltype(njc)::value;
+            constexpr bool more = decltype(morec)::value != 0;
             read_a();
             // the wave's A region is free again once its reads have returned
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            issue_b(sb, 1);
-            compute_half(std::integral_constant<int, 0>{}, njc, sb, more);
-            // the second half of B has landed (the younger weight loads may still be on their way)
-            if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kAFirst) : "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            if (more) {
-                issue_b(sb + 1u, 0);
-                issue_bt(sb + 1u);
+            if constexpr (more) {
+                issue_phase(sb + 1u, 0, (sb + 1u) & 1u);
                 issue_yd(sb + 1u);
+                // fewer operands than weight loads: the rest of the loads in front
+                gemm_static_for<4 * NJ, kALoads>([&](auto lc) __attribute__((always_inline)) { issue_a_one(decltype(lc)::value, sb + 1u); });
             }
-            compute_half(std::integral_constant<int, 1>{}, njc, sb, more);
+            constexpr int kBeside = !more ? 0 : 4 * NJ < kALoads ? 4 * NJ : kALoads;
+            compute_phase(njc, I0{}, I0{}, std::integral_constant<int, kBeside>{}, sb & 1u, sb);
             // everything this wave fetched for the next super-block has landed before the others
             // may read it
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-        }
-    };
-    // the number of column groups that hold a real column picks the instantiation
-    if constexpr (kGemmCG == 1) {
-        main_loop(std::integral_constant<int, 1>{});
-    } else {
+        };
+        // up to 64 columns: one phase per super-block, the buffers alternate by super-block
+        auto loop_one_phase = [&](auto njc) {
+            uint32_t sb = 0;
+            for (; sb + 1u < p.n_sb; sb++) step_one_phase(njc, I1{}, sb);
+            step_one_phase(njc, I0{}, sb);
+        };
+        auto step_two_phases = [&](auto njc, auto morec, const uint32_t sb) __attribute__((always_inline)) {
+            constexpr int NJ2 = decltype(njc)::value - 4;
+            constexpr bool more = decltype(morec)::value != 0;
+            read_a();
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            issue_phase(sb, 1, 1u);
+            compute_phase(std::integral_constant<int, 4>{}, I0{}, I0{}, std::integral_constant<int, more ? kALoads : 0>{}, 0u, sb);
+            // the second phase's columns have landed (the younger weight loads may still be on
+            // their way)
+            if constexpr (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kALoads) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if constexpr (more) {
+                issue_phase(sb + 1u, 0, 0u);
+                issue_yd(sb + 1u);
+            }
+            compute_phase(std::integral_constant<int, NJ2>{}, std::integral_constant<int, 4>{}, I0{}, I0{}, 1u, sb);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        };
+        // more: columns 0..63 from buffer 0, then 64.. from buffer 1
+        auto loop_two_phases = [&](auto njc) {
+            uint32_t sb = 0;
+            for (; sb + 1u < p.n_sb; sb++) step_two_phases(njc, I1{}, sb);
+            step_two_phases(njc, I0{}, sb);
+        };
         switch (nj) {
-            case 1: main_loop(std::integral_constant<int, 1>{}); break;
-            case 2: main_loop(std::integral_constant<int, 2>{}); break;
-            case 3: main_loop(std::integral_constant<int, 3>{}); break;
-            case 4: main_loop(std::integral_constant<int, 4>{}); break;
-            case 5: main_loop(std::integral_constant<int, 5>{}); break;
-            case 6: main_loop(std::integral_constant<int, 6>{}); break;
-            case 7: main_loop(std::integral_constant<int, 7>{}); break;
-            default: main_loop(std::integral_constant<int, 8>{}); break;
+            case 1: loop_one_phase(std::integral_constant<int, 1>{}); break;
+            case 2: loop_one_phase(std::integral_constant<int, 2>{}); break;
+            case 3: loop_one_phase(std::integral_constant<int, 3>{}); break;
+            case 4: loop_one_phase(std::integral_constant<int, 4>{}); break;
+            case 5: loop_two_phases(std::integral_constant<int, 5>{}); break;
+            case 6: loop_two_phases(std::integral_constant<int, 6>{}); break;
+            case 7: loop_two_phases(std::integral_constant<int, 7>{}); break;
+            default: loop_two_phases(std::integral_constant<int, 8>{}); break;
         }
+    } else {
+        // ---- the narrow tile: B by half super-blocks ------------------------------------
+        const uint32_t b_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 2048u);
+        const uint32_t bt_lds = __builtin_amdgcn_readfirstlane(lds0 + kTailsOff + wave * 2048u);
+        uint32_t b_fetch[2];   // column 16 w + 8 ii + l8, chunk c8 = lane % 8 ^ l8 of a 128-byte run
+    #pragma unroll
+        for (int ii = 0; ii < 2; ii++)
+            b_fetch[ii] = s_src[(wave * 16u + ii * 8u + l8) & (uint32_t)(MT - 1)] * p.act_row_bytes + c8 * 16u;
+        // a wave whose 16 columns lie past the end of a short group fetches nothing (nobody reads
+        // them: the column loop stops at the last group that holds a real column)
+        const bool b_live = wave * 16u < cnt;
+        auto issue_b = [&](uint32_t sb, uint32_t h) {  // the heads of half h, into heads buffer h
+            if (!b_live) return;
+            const uint8_t *src = p.act + (sb * kStaged6Bytes + h * 128u);
+    #pragma unroll
+            for (int ii = 0; ii < 2; ii++)
+                lds_dma16(b_lds + h * kHeadsBytes + (uint32_t)(ii * 1024), src, b_fetch[ii]);
+        };
+        auto issue_bt = [&](uint32_t sb) {  // the tails of both halves, into tails buffer sb % 2
+            if (!b_live) return;
+            const uint8_t *src = p.act + (sb * kStaged6Bytes + 256u);
+            lds_dma16(bt_lds + (sb & 1u) * kTailsBytes, src, b_fetch[0]);
+            lds_dma16(bt_lds + (sb & 1u) * kTailsBytes + 1024u, src, b_fetch[1] ^ 16u);
+        };
+
+        issue_b(0, 0);
+        issue_bt(0);
+        issue_yd(0);
+    #pragma unroll
+        for (int r = 0; r < kGemmRF; r++)
+    #pragma unroll
+            for (int m = 0; m < 2; m++)
+    #pragma unroll
+                for (int j = 0; j < kGemmCG; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+
+        const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
+        // One half super-block with NJ column groups (compile-time, so the code below is one
+        // straight line): for every group, the two pieces (high and low plane) against the wave's
+        // four fragments, then the fold acc += d * c -- placed right before each fragment's
+        // temporary is overwritten by the next group's first piece.  The next piece's B operand is
+        // requested from LDS one piece ahead of its use (deeper changes nothing).  Empty asm
+        // statements pin that order; they emit no instruction, so the compiler still sees every
+        // real one and keeps its hazards.  Left alone it hoists every LDS read of the half to its
+        // top, which overflows the registers, pulls each fold up to the instruction that produces
+        // its input, where it waits, and with the group count as a run-time condition waits for
+        // each operand right after requesting it (layer at T=4096: 4.5 -> 4.0 ms).
+    #define DSX_PIN() asm volatile("" ::: "memory")
+        auto compute_half = [&](auto hc, auto njc, const uint32_t sb, const bool more) {
+            constexpr int h = decltype(hc)::value;
+            constexpr int NJ = decltype(njc)::value;
+            const uint8_t *half = tiles + h * kHeadsBytes;
+            const uint8_t *tails = tiles + kTailsOff + (sb & 1u) * kTailsBytes;
+            const float *yds = s_yd + ((sb >> 2) & 1u) * (uint32_t)(kYdBytes / 4) + (sb & 3u);
+            // the operand of (column group j, plane q): 16 bytes of head, 8 of tail
+            auto load_piece = [&](int j, int q) -> v8i {
+                const uint32_t cb = (((uint32_t)(2 * j) + (n16 >> 3)) * 1024u + sw) ^ ((uint32_t)q * 64u);
+                const uint4 hd = *(const uint4 *)(half + cb);
+                const uint2 tl = *(const uint2 *)(tails + (uint32_t)j * 2048u +
+                                                  (bt_rd ^ ((uint32_t)q * 32u) ^ ((uint32_t)h * 64u)));
+                return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
+            };
+            v4f c[kGemmRF][2];
+            // piece p = 2 j + q alternates between two operand registers
+            constexpr int NP = 2 * NJ;
+            v8i ring[2];
+            ring[0] = load_piece(0, 0);
+            float yd_prev = 0.0f, yd = 0.0f;
+            DSX_PIN();
+    #pragma unroll
+            for (int pc = 0; pc < NP; pc++) {
+                const int j = pc >> 1, q = pc & 1;
+                if (q == 0) yd = yds[(j * 16u + n16) * 4u];
+                if (pc + 1 < NP) ring[(pc + 1) & 1] = load_piece((pc + 1) >> 1, (pc + 1) & 1);
+                DSX_PIN();
+                v8i &bq = ring[pc & 1];
+                asm volatile("" : "+v"(bq));  // the products with this piece stay behind the request above
+    #pragma unroll
+                for (int r = 0; r < kGemmRF; r++)
+    #pragma unroll
+                    for (int m = 0; m < 2; m++) {
+                        const GemmAFrag &w = a_cur[r][m];
+                        const uint4 &aw = h == 0 ? w.a0 : w.a1;
+                        const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
+                        if (q == 0) {
+                            if (j > 0) {
+                                asm volatile("" : "+v"(c[r][m]));
+                                v4f &a = acc[r][m][j > 0 ? j - 1 : 0];
+                                a.x = fmaf(yd_prev, c[r][m].x, a.x);
+                                a.y = fmaf(yd_prev, c[r][m].y, a.y);
+                                a.z = fmaf(yd_prev, c[r][m].z, a.z);
+                                a.w = fmaf(yd_prev, c[r][m].w, a.w);
+                                asm volatile("" : "+v"(a));
+                            }
+                            c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 2, h, (int)w.sc, 0, kScaleB6High);
+                        } else {
+                            c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                av, bq, c[r][m], 4, 2, h, (int)w.sc, 0, kScaleB6Low);
+                        }
+                    }
+                if (q == 1) yd_prev = yd;
+                // the next super-block's weights, a load or two behind each piece's products: a
+                // request that has to wait for room in the memory pipeline then holds back nothing
+                // that the matrix pipe does not already have
+                {
+                    constexpr int kFrom = h == 0 ? 0 : kAFirst, kCnt = h == 0 ? kAFirst : kALoads - kAFirst;
+                    // behind the first pieces of a half: 8 of the 10 in the first half, one per piece (a
+                    // few per cent faster than 6 + 4 and than all 10 at once, measured at 4096 tokens)
+                    constexpr int kSpan = h == 0 ? (NP < 8 ? NP : 8) : (NP + 1) / 2;
+                    const int lo = pc * kCnt / kSpan, hi = (pc + 1) * kCnt / kSpan;
+                    if (pc < kSpan && more) {
+                        // literal indices: the load's registers are picked at compile time
+                        if (0 < kCnt && lo <= 0 && 0 < hi) issue_a_one(kFrom + 0, sb + 1u);
+                        if (1 < kCnt && lo <= 1 && 1 < hi) issue_a_one(kFrom + 1, sb + 1u);
+                        if (2 < kCnt && lo <= 2 && 2 < hi) issue_a_one(kFrom + 2, sb + 1u);
+                        if (3 < kCnt && lo <= 3 && 3 < hi) issue_a_one(kFrom + 3, sb + 1u);
+                        if (4 < kCnt && lo <= 4 && 4 < hi) issue_a_one(kFrom + 4, sb + 1u);
+                        if (5 < kCnt && lo <= 5 && 5 < hi) issue_a_one(kFrom + 5, sb + 1u);
+                        if (6 < kCnt && lo <= 6 && 6 < hi) issue_a_one(kFrom + 6, sb + 1u);
+                        if (7 < kCnt && lo <= 7 && 7 < hi) issue_a_one(kFrom + 7, sb + 1u);
+                        if (8 < kCnt && lo <= 8 && 8 < hi) issue_a_one(kFrom + 8, sb + 1u);
+                        if (9 < kCnt && lo <= 9 && 9 < hi) issue_a_one(kFrom + 9, sb + 1u);
+                    }
+                }
+            }
+            // fold the last group
+    #pragma unroll
+            for (int r = 0; r < kGemmRF; r++)
+    #pragma unroll
+                for (int m = 0; m < 2; m++) {
+                    v4f &a = acc[r][m][NJ - 1];
+                    a.x = fmaf(yd_prev, c[r][m].x, a.x);
+                    a.y = fmaf(yd_prev, c[r][m].y, a.y);
+                    a.z = fmaf(yd_prev, c[r][m].z, a.z);
+                    a.w = fmaf(yd_prev, c[r][m].w, a.w);
+                }
+        };
+    #undef DSX_PIN
+
+        auto main_loop = [&](auto njc) {
+            for (uint32_t sb = 0; sb < p.n_sb; sb++) {
+                const bool more = sb + 1u < p.n_sb;
+                read_a();
+                // the wave's A region is free again once its reads have returned
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue_b(sb, 1);
+                compute_half(std::integral_constant<int, 0>{}, njc, sb, more);
+                // the second half of B has landed (the younger weight loads may still be on their way)
+                if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kAFirst) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (more) {
+                    issue_b(sb + 1u, 0);
+                    issue_bt(sb + 1u);
+                    issue_yd(sb + 1u);
+                }
+                compute_half(std::integral_constant<int, 1>{}, njc, sb, more);
+                // everything this wave fetched for the next super-block has landed before the others
+                // may read it
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
+        };
+        // the number of column groups that hold a real column picks the instantiation
+        if constexpr (kGemmCG == 1) {
+            main_loop(std::integral_constant<int, 1>{});
+        } else {
+            switch (nj) {
+                case 1: main_loop(std::integral_constant<int, 1>{}); break;
+                case 2: main_loop(std::integral_constant<int, 2>{}); break;
+                case 3: main_loop(std::integral_constant<int, 3>{}); break;
+                case 4: main_loop(std::integral_constant<int, 4>{}); break;
+                case 5: main_loop(std::integral_constant<int, 5>{}); break;
+                case 6: main_loop(std::integral_constant<int, 6>{}); break;
+                case 7: main_loop(std::integral_constant<int, 7>{}); break;
+                default: main_loop(std::integral_constant<int, 8>{}); break;
+            }
+        }
+
     }
 
     // ---- epilogue ---------------------------------------------------------------------
