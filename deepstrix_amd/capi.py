@@ -48,6 +48,13 @@ class LayerDesc(C.Structure):
     ]
 
 
+class HcPostDesc(C.Structure):
+    """dsx_hc_post_desc (include/dsx_moe.h)."""
+    _fields_ = [("out_hc", C.c_void_p), ("residual_hc", C.c_void_p), ("post", C.c_void_p),
+                ("comb", C.c_void_p), ("n_hc", C.c_uint32), ("post_stride", C.c_uint32),
+                ("comb_stride", C.c_uint32)]
+
+
 _vp, _u32, _u64, _f32, _int, _sz = C.c_void_p, C.c_uint32, C.c_uint64, C.c_float, C.c_int, C.c_size_t
 
 # name -> (restype, argtypes); every symbol include/dsx_moe.h declares
@@ -97,6 +104,8 @@ SIGNATURES = {
     "dsx_moe_block_forward_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _u32, _vp, _sz]),
     "dsx_moe_layer_forward_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp]),
     "dsx_moe_layer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _sz, _vp, _vp, _vp, _vp]),
+    "dsx_moe_layer_forward_hc": (_int, [_vp, _vp, C.POINTER(HcPostDesc), _vp, _vp, _u32, _vp, _sz, _vp, _vp, _vp, _vp]),
+    "dsx_hc_post": (_int, [_vp, C.POINTER(HcPostDesc), _vp, _vp, _vp, _u32, _u32]),
 }
 
 _lib = None

@@ -623,15 +623,16 @@ int dsx_moe_down_by_expert(dsx_stream_t stream, int dtype, float *partials, cons
 }
 
 static int reduce_impl(hipStream_t st, float *out, const float *partials, const int32_t *selected,
-                       const float *add, uint32_t n_used, uint32_t n_rows, uint32_t b) {
+                       const float *add, uint32_t n_used, uint32_t n_rows, uint32_t b,
+                       const HcPost &hc = HcPost{}) {
     if (b == 0) return DSX_OK;
-    if (!out || !partials) return fail(DSX_ERR_INVALID_ARG, "moe_reduce_partials: null pointer");
+    if ((!out && !hc.n_hc) || !partials) return fail(DSX_ERR_INVALID_ARG, "moe_reduce_partials: null pointer");
     if (n_rows == 0 || n_rows % 4 != 0 || !aligned(out, 16) || !aligned(partials, 16) ||
         (add && !aligned(add, 16)))
         return fail(DSX_ERR_SHAPE, "moe_reduce_partials: n_rows=%u must be a multiple of 4, buffers 16-byte aligned", n_rows);
     const uint64_t n4 = (uint64_t)b * (n_rows / 4);
     hipLaunchKernelGGL(k_reduce_partials, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, st, out,
-                       partials, selected, add, n_used, n_rows, b);
+                       partials, selected, add, n_used, n_rows, b, hc);
     return launched("moe_reduce_partials");
 }
 
@@ -673,6 +674,40 @@ int dsx_router_logits(dsx_stream_t stream, float *logits, const float *router_w,
 int dsx_router_logits_f16(dsx_stream_t stream, float *logits, const uint16_t *router_w,
                           const float *x, uint32_t n_expert, uint32_t hidden, uint32_t n_tokens) {
     return router_logits_impl(stream, logits, (const __half *)router_w, x, n_expert, hidden, n_tokens);
+}
+
+// ---- hyper-connection combine --------------------------------------------------------------
+// Checks a caller's descriptor and turns it into the kernels' (0 = ok).
+static int hc_post_args(const char *who, const dsx_hc_post_desc *d, uint32_t n_embd, HcPost *out) {
+    if (!d || !d->out_hc || !d->residual_hc || !d->post || !d->comb)
+        return fail(DSX_ERR_INVALID_ARG, "%s: null pointer in the hc_post descriptor", who);
+    if (d->n_hc == 0 || d->n_hc > kMaxHc)
+        return fail(DSX_ERR_INVALID_ARG, "%s: n_hc=%u not in 1..%u", who, d->n_hc, kMaxHc);
+    if (n_embd == 0 || n_embd % 4 != 0 || !aligned(d->out_hc, 16) || !aligned(d->residual_hc, 16))
+        return fail(DSX_ERR_SHAPE, "%s: n_embd=%u must be a multiple of 4, out_hc / residual_hc 16-byte aligned", who, n_embd);
+    *out = HcPost{d->out_hc, d->residual_hc, d->post, d->comb, d->n_hc, d->post_stride, d->comb_stride};
+    return DSX_OK;
+}
+
+static int add_rows_impl(hipStream_t st, float *out, const float *a, const float *b, const float *c,
+                         uint32_t n_embd, uint32_t n_tokens, const HcPost &hc) {
+    const uint64_t n4 = (uint64_t)n_tokens * (n_embd / 4u);
+    hipLaunchKernelGGL(k_add_rows, dim3((uint32_t)((n4 + 255u) / 256u)), dim3(256), 0, st, out, a, b, c,
+                       n_embd, n_tokens, hc);
+    return launched("add_rows");
+}
+
+int dsx_hc_post(dsx_stream_t stream, const dsx_hc_post_desc *desc, const float *block_out,
+                const float *add1, const float *add2, uint32_t n_embd, uint32_t b) {
+    if (b == 0) return DSX_OK;
+    if (!block_out) return fail(DSX_ERR_INVALID_ARG, "hc_post: null block_out");
+    if (add2 && !add1) return fail(DSX_ERR_INVALID_ARG, "hc_post: add2 without add1");
+    HcPost hc{};
+    if (int rc = hc_post_args("hc_post", desc, n_embd, &hc)) return rc;
+    if (!aligned(block_out, 16) || (add1 && !aligned(add1, 16)) || (add2 && !aligned(add2, 16)))
+        return fail(DSX_ERR_SHAPE, "hc_post: block_out / add1 / add2 must be 16-byte aligned");
+    if ((uint64_t)b * (n_embd / 4u) > 0xFFFFFFFFull * 256ull) return fail(DSX_ERR_INVALID_ARG, "hc_post: too many rows");
+    return add_rows_impl(S(stream), nullptr, block_out, add1, add2, n_embd, b, hc);
 }
 
 // ---- element-wise -----------------------------------------------------------------------

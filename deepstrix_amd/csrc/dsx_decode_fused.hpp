@@ -75,6 +75,7 @@ struct DecodeFusedParams {
     float *out;                      // [n_tokens, hidden]
     const float *residual;           // [n_tokens, hidden] or null; may alias out
     const float *shared_rows;        // [n_tokens, hidden] or null: a shared expert computed before the launch
+    HcPost hc;                       // n_hc != 0: the result goes through the hyper-connection combine instead of to out
     uint32_t *slot_done;             // [n_tokens, n_slots], zero on entry
     uint32_t *ready;                 // [n_tokens, n_slots, kDfFan] flags kDfFanStride words apart, zero on entry
     uint32_t dn_early;               // super-blocks of a down item's weights requested before its mid row is checked
@@ -590,7 +591,8 @@ __device__ __forceinline__ void df_combine(const DecodeFusedParams &p, uint32_t 
             if ((uint32_t)q < p.n_slots) s += (uint32_t)q == own_slot ? own : v[q];
         if (p.shared_rows) s += p.shared_rows[o];
         if (p.residual) s += p.residual[o];
-        p.out[o] = s;
+        if (p.hc.n_hc) hc_post_store(p.hc, t, row0 + (lane & 15u), p.hidden, s);
+        else p.out[o] = s;
     }
 }
 

@@ -306,4 +306,55 @@ __device__ __forceinline__ float swiglu_clamp(float g, float u, float clamp, flo
     return g * sig * u * ew;
 }
 
+// ---- the hyper-connection combine behind a sublayer --------------------------------------------
+// out_hc[t, dst, d] = block[t, d] * post[t, dst] + sum_src comb[t, dst + src * n_hc] * residual_hc[t, src, d]
+// (crates/v4flash-kernels/kernels/hc_post.hip:15-34, batched :40-64; sums in f32, src ascending,
+// products rounded before they are added).  post / comb of token t start post_stride / comb_stride
+// floats behind those of token t - 1, so that one descriptor covers separate arrays
+// ([b, n_hc] and [b, n_hc, n_hc]) and the reference's packed "split" rows alike
+// (hc_post.hip:66-98: post at n_w, comb at n_w + n_hc of a row of n_w + n_hc + n_hc * n_hc).
+// n_hc == 0: no combine.
+constexpr uint32_t kMaxHc = 8;
+struct HcPost {
+    float *out_hc;              // [b, n_hc, n_embd]
+    const float *residual_hc;   // [b, n_hc, n_embd]
+    const float *post, *comb;
+    uint32_t n_hc, post_stride, comb_stride;
+};
+// one value (token t, element d of n_embd)
+__device__ __forceinline__ void hc_post_store(const HcPost &h, uint64_t t, uint32_t d, uint32_t n_embd, float block) {
+    const float *post = h.post + t * h.post_stride, *comb = h.comb + t * h.comb_stride;
+    const float *res = h.residual_hc + t * h.n_hc * n_embd + d;
+    float r[kMaxHc];
+#pragma unroll
+    for (uint32_t s = 0; s < kMaxHc; s++) r[s] = s < h.n_hc ? res[(uint64_t)s * n_embd] : 0.0f;
+    for (uint32_t dst = 0; dst < h.n_hc; dst++) {
+        float acc = block * post[dst];
+#pragma unroll
+        for (uint32_t s = 0; s < kMaxHc; s++)
+            if (s < h.n_hc) acc += comb[dst + s * h.n_hc] * r[s];
+        h.out_hc[(t * h.n_hc + dst) * n_embd + d] = acc;
+    }
+}
+// four consecutive values (d a multiple of 4)
+__device__ __forceinline__ void hc_post_store4(const HcPost &h, uint64_t t, uint32_t d, uint32_t n_embd, float4 block) {
+    const float *post = h.post + t * h.post_stride, *comb = h.comb + t * h.comb_stride;
+    const float *res = h.residual_hc + t * h.n_hc * n_embd + d;
+    float4 r[kMaxHc];
+#pragma unroll
+    for (uint32_t s = 0; s < kMaxHc; s++)
+        r[s] = s < h.n_hc ? *(const float4 *)(res + (uint64_t)s * n_embd) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t dst = 0; dst < h.n_hc; dst++) {
+        const float pd = post[dst];
+        float4 acc = make_float4(block.x * pd, block.y * pd, block.z * pd, block.w * pd);
+#pragma unroll
+        for (uint32_t s = 0; s < kMaxHc; s++)
+            if (s < h.n_hc) {
+                const float c = comb[dst + s * h.n_hc];
+                acc.x += c * r[s].x; acc.y += c * r[s].y; acc.z += c * r[s].z; acc.w += c * r[s].w;
+            }
+        *(float4 *)(h.out_hc + (t * h.n_hc + dst) * n_embd + d) = acc;
+    }
+}
+
 }  // namespace dsx

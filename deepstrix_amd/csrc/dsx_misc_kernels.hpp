@@ -798,12 +798,13 @@ __global__ __launch_bounds__(256) void k_group_scatter(int32_t *__restrict__ mem
 // `selected` (nullable): slots with a negative pick are skipped.
 // `add` (nullable): added last (the shared expert, crates/v4flash-kernels/kernels/vec_add.hip:6-13).
 // ---------------------------------------------------------------------------------------
+// `hc` (n_hc != 0): the sum is not stored but goes through the hyper-connection combine.
 __global__ __launch_bounds__(256) void k_reduce_partials(float *__restrict__ out,
                                                          const float *__restrict__ partials,
                                                          const int32_t *__restrict__ selected,
                                                          const float *__restrict__ add,
                                                          uint32_t n_used, uint32_t n_rows,
-                                                         uint32_t b) {
+                                                         uint32_t b, const HcPost hc) {
     const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;  // float4 index
     const uint64_t per_row = n_rows / 4u;
     if (i >= (uint64_t)b * per_row) return;
@@ -824,7 +825,8 @@ __global__ __launch_bounds__(256) void k_reduce_partials(float *__restrict__ out
         acc.z += v.z;
         acc.w += v.w;
     }
-    *(float4 *)(out + t * n_rows + c * 4u) = acc;
+    if (hc.n_hc) hc_post_store4(hc, t, (uint32_t)c * 4u, n_rows, acc);
+    else *(float4 *)(out + t * n_rows + c * 4u) = acc;
 }
 
 // crates/v4flash-kernels/kernels/vec_add.hip:6-13
@@ -835,20 +837,33 @@ __global__ __launch_bounds__(256) void k_vec_add_inplace(float *__restrict__ out
     if (i < n) out[i] += rhs[i];
 }
 
-// out = (a + b) + c  (c may be null; out may alias any of them): the routed experts' rows, a shared
-// expert computed beside them and the residual, in the order the reference adds them
-// (crates/v4flash-kernels/src/het/forward_prefill.rs:12227-12232).  n is a multiple of 4.
+// out = (a + b) + c  (b, c may be null; out may alias any of them): the routed experts' rows, a
+// shared expert computed beside them and the residual, in the order the reference adds them
+// (crates/v4flash-kernels/src/het/forward_prefill.rs:12227-12232; with both addends the block
+// value of hc_post_from_split_batched_add2, crates/v4flash-kernels/kernels/hc_post.hip:100-141).
+// `hc` (n_hc != 0): the sum goes through the hyper-connection combine instead of to `out`.
+// n_embd is a multiple of 4.
 __global__ __launch_bounds__(256) void k_add_rows(float *out, const float *a, const float *b,
-                                                  const float *c, uint64_t n4) {
+                                                  const float *c, uint32_t n_embd, uint32_t n_tokens,
+                                                  const HcPost hc) {
     const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-    if (i >= n4) return;
-    const float4 va = ((const float4 *)a)[i], vb = ((const float4 *)b)[i];
-    float4 s = make_float4(va.x + vb.x, va.y + vb.y, va.z + vb.z, va.w + vb.w);
+    const uint64_t per_row = n_embd / 4u;
+    if (i >= (uint64_t)n_tokens * per_row) return;
+    float4 s = ((const float4 *)a)[i];
+    if (b) {
+        const float4 vb = ((const float4 *)b)[i];
+        s.x += vb.x; s.y += vb.y; s.z += vb.z; s.w += vb.w;
+    }
     if (c) {
         const float4 vc = ((const float4 *)c)[i];
         s.x += vc.x; s.y += vc.y; s.z += vc.z; s.w += vc.w;
     }
-    ((float4 *)out)[i] = s;
+    if (hc.n_hc) {
+        const uint64_t t = i / per_row;
+        hc_post_store4(hc, t, (uint32_t)(i - t * per_row) * 4u, n_embd, s);
+    } else {
+        ((float4 *)out)[i] = s;
+    }
 }
 
 // crates/v4flash-kernels/kernels/swiglu_clamp_weighted.hip:16-37

@@ -157,6 +157,24 @@ def vec_add_inplace(out, rhs, n):
     check(lib().dsx_vec_add_inplace(_stream(), _p(out), _p(rhs), n))
 
 
+def hc_post_desc(out_hc, residual_hc, post, comb, n_hc, post_stride=None, comb_stride=None) -> capi.HcPostDesc:
+    """dsx_hc_post_desc over device tensors; strides default to separate [b, n_hc] / [b, n_hc, n_hc]
+    arrays (pass both as n_w + n_hc + n_hc * n_hc for views into the engine's packed split rows)."""
+    d = capi.HcPostDesc()
+    d.out_hc, d.residual_hc, d.post, d.comb = _p(out_hc), _p(residual_hc), _p(post), _p(comb)
+    d.n_hc = n_hc
+    d.post_stride = n_hc if post_stride is None else post_stride
+    d.comb_stride = n_hc * n_hc if comb_stride is None else comb_stride
+    return d
+
+
+def hc_post(desc: capi.HcPostDesc, block_out, n_embd, b, add1=None, add2=None):
+    """HcPost::launch* (crates/v4flash-kernels/kernels/hc_post.hip:15-141)."""
+    import ctypes as C
+    capi.init()
+    check(lib().dsx_hc_post(_stream(), C.byref(desc), _p(block_out), _p(add1), _p(add2), n_embd, b))
+
+
 def rms_norm(out, x, weight, n, eps, rows):
     capi.init()
     check(lib().dsx_rms_norm(_stream(), _p(out), _p(x), _p(weight), n, eps, rows))

@@ -194,6 +194,25 @@ class MoeLayer:
             return out, sel_out, w_out
         return out
 
+    def run_hc(self, x: torch.Tensor, logits: Optional[torch.Tensor], hc, selected_in=None,
+               weights_in=None, want_routing=False):
+        """`run` whose result goes through the hyper-connection combine `hc` (a capi.HcPostDesc,
+        see dispatch.hc_post_desc) instead of to an output buffer (dsx_moe_layer_forward_hc)."""
+        T = x.shape[0]
+        if T > self.max_tokens:
+            raise ValueError(f"{T} tokens > max_tokens={self.max_tokens}")
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        sel_out = w_out = None
+        if want_routing:
+            sel_out = torch.empty((T, self.w.n_used), dtype=torch.int32, device=x.device)
+            w_out = torch.empty((T, self.w.n_used), dtype=torch.float32, device=x.device)
+        p = lambda t: None if t is None else t.data_ptr()
+        check(lib().dsx_moe_layer_forward_hc(
+            self._h, torch.cuda.current_stream().cuda_stream, C.byref(hc), p(x), p(logits), T,
+            p(self.workspace), self.workspace_bytes, p(sel_out), p(w_out), p(selected_in),
+            p(weights_in)))
+        return (sel_out, w_out) if want_routing else None
+
     def run_noalloc(self, x: torch.Tensor, logits: Optional[torch.Tensor], out: torch.Tensor,
                     selected_in=None, weights_in=None, selected_out=None, weights_out=None):
         """`run` through dsx_moe_layer_forward_noalloc: the library's built-in scratch array

@@ -215,6 +215,31 @@ int dsx_dense_ffn(dsx_stream_t stream, int gate_fmt, int up_fmt, int down_fmt, f
 /* ---- element-wise ----------------------------------------------------------
  * VecAddInplace::launch (crates/v4flash-kernels/src/ffn.rs:135-153). */
 int dsx_vec_add_inplace(dsx_stream_t stream, float *out, const float *rhs, uint64_t n);
+
+/* ---- hyper-connection combine behind the FFN ----------------------------------
+ * HcPost::launch / launch_batched / launch_from_split* (kernels
+ * crates/v4flash-kernels/kernels/hc_post.hip:15-34, 40-64, 66-98, 100-141; call site
+ * crates/v4flash-kernels/src/het/forward_layer.rs:3126-3133, right behind the vec_add that adds
+ * the shared expert):
+ *   out_hc[t, dst, d] = block[t, d] * post[t, dst]
+ *                       + sum_src comb[t, dst + src * n_hc] * residual_hc[t, src, d]
+ * in f32, src ascending.  post / comb of token t start post_stride / comb_stride floats behind
+ * those of token t - 1: separate arrays ([b, n_hc], [b, n_hc, n_hc]: strides n_hc, n_hc * n_hc)
+ * and the engine's packed "split" rows (post = split + n_w, comb = split + n_w + n_hc, both
+ * strides n_w + n_hc + n_hc * n_hc) are the same descriptor.  out_hc may be residual_hc itself
+ * (every element's inputs are read before its outputs are written).  n_hc <= 8. */
+typedef struct dsx_hc_post_desc {
+    float *out_hc;             /* [b, n_hc, n_embd] */
+    const float *residual_hc;  /* [b, n_hc, n_embd] */
+    const float *post;         /* n_hc per token */
+    const float *comb;         /* n_hc * n_hc per token, addressed [dst + src * n_hc] */
+    uint32_t n_hc, post_stride, comb_stride;
+} dsx_hc_post_desc;
+/* block[t, d] = block_out[t, d] (+ add1[t, d] (+ add2[t, d])): with both addends the block value
+ * of hc_post_from_split_batched_add2, (block_out + add1) + add2; add1 / add2 may be NULL (add2
+ * only with add1).  block_out is not written. */
+int dsx_hc_post(dsx_stream_t stream, const dsx_hc_post_desc *desc, const float *block_out,
+                const float *add1, const float *add2, uint32_t n_embd, uint32_t b);
 /* RmsNorm batched (crates/v4flash-kernels/src/rms_norm.rs; kernels/rms_norm.hip:52-). */
 int dsx_rms_norm(dsx_stream_t stream, float *out, const float *x, const float *weight,
                  uint32_t n, float eps, uint32_t rows);
@@ -364,6 +389,15 @@ int dsx_moe_layer_forward(dsx_moe_layer *layer, dsx_stream_t stream, float *out,
                           size_t workspace_bytes, int32_t *selected_out, float *weights_out,
                           const int32_t *selected_in, const float *weights_in);
 
+/* dsx_moe_layer_forward whose result goes straight through the hyper-connection combine
+ * (dsx_hc_post above with block = the layer's output, n_embd = hidden) instead of to an output
+ * buffer: the kernel that sums a token's slots and the shared expert applies it while it stores
+ * -- the reference's vec_add + hc_post pair (crates/v4flash-kernels/src/het/forward_layer.rs:3126-3133)
+ * without the launches and without the round trip of the layer output through memory. */
+int dsx_moe_layer_forward_hc(dsx_moe_layer *layer, dsx_stream_t stream, const dsx_hc_post_desc *hc,
+                             const float *x, const float *logits, uint32_t n_tokens, void *workspace,
+                             size_t workspace_bytes, int32_t *selected_out, float *weights_out,
+                             const int32_t *selected_in, const float *weights_in);
 /* dsx_moe_layer_forward without a workspace argument.  No counterpart in the reference: it is
  * for callers that cannot allocate device memory at all (code under HIP graph capture that owns
  * no buffers, tight serving loops, harnesses that forbid hipMalloc).  The scratch is a fixed

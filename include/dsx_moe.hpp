@@ -313,6 +313,52 @@ struct MoeGroupBuilder {
     }
 };
 
+// ---- HcPost (crates/v4flash-kernels/src/head.rs:269-500) ---------------------------------------
+// The hyper-connection combine behind the FFN; the names are the reference wrapper's.
+struct HcPost {
+    // launch / launch_batched (head.rs:286-345): separate post [b, n_hc] and comb [b, n_hc, n_hc]
+    static Status launch_batched(const Stream &s, Out<float> out_hc, In<float> block_out, In<float> residual_hc,
+                                 In<float> post, In<float> comb, uint32_t n_embd, uint32_t n_hc, uint32_t batch) {
+        DSX_TRY(detail::need("hc_post out_hc", out_hc.len(), (size_t)batch * n_hc * n_embd));
+        DSX_TRY(detail::need("hc_post block_out", block_out.len(), (size_t)batch * n_embd));
+        DSX_TRY(detail::need("hc_post residual_hc", residual_hc.len(), (size_t)batch * n_hc * n_embd));
+        DSX_TRY(detail::need("hc_post post", post.len(), (size_t)batch * n_hc));
+        DSX_TRY(detail::need("hc_post comb", comb.len(), (size_t)batch * n_hc * n_hc));
+        const dsx_hc_post_desc d{out_hc.ptr(), residual_hc.ptr(), post.ptr(), comb.ptr(), n_hc, n_hc, n_hc * n_hc};
+        return Status::from_c(dsx_hc_post(s.raw(), &d, block_out.ptr(), nullptr, nullptr, n_embd, batch),
+                              "HcPost::launch_batched");
+    }
+    static Status launch(const Stream &s, Out<float> out_hc, In<float> block_out, In<float> residual_hc,
+                         In<float> post, In<float> comb, uint32_t n_embd, uint32_t n_hc) {
+        return launch_batched(s, out_hc, block_out, residual_hc, post, comb, n_embd, n_hc, 1u);
+    }
+    // launch_from_split_batched / _add / _add2 (head.rs:347-455): post and comb inside the packed
+    // rows split[batch, n_w + n_hc + n_hc * n_hc]; add1 / add2 may be empty (add2 only with add1):
+    // block = (block_out + add1) + add2
+    static Status launch_from_split_batched_add2(const Stream &s, Out<float> out_hc, In<float> block_out,
+                                                 In<float> add1, In<float> add2, In<float> residual_hc,
+                                                 In<float> split, uint32_t n_w, uint32_t n_embd, uint32_t n_hc,
+                                                 uint32_t batch) {
+        const uint32_t stride = n_w + n_hc + n_hc * n_hc;
+        DSX_TRY(detail::need("hc_post out_hc", out_hc.len(), (size_t)batch * n_hc * n_embd));
+        DSX_TRY(detail::need("hc_post block_out", block_out.len(), (size_t)batch * n_embd));
+        DSX_TRY(detail::need("hc_post residual_hc", residual_hc.len(), (size_t)batch * n_hc * n_embd));
+        DSX_TRY(detail::need("hc_post split", split.len(), (size_t)batch * stride));
+        if (!add1.empty()) DSX_TRY(detail::need("hc_post add1", add1.len(), (size_t)batch * n_embd));
+        if (!add2.empty()) DSX_TRY(detail::need("hc_post add2", add2.len(), (size_t)batch * n_embd));
+        const dsx_hc_post_desc d{out_hc.ptr(), residual_hc.ptr(), split.ptr() + n_w, split.ptr() + n_w + n_hc,
+                                 n_hc, stride, stride};
+        return Status::from_c(dsx_hc_post(s.raw(), &d, block_out.ptr(), add1.ptr(), add2.ptr(), n_embd, batch),
+                              "HcPost::launch_from_split_batched");
+    }
+    static Status launch_from_split_batched(const Stream &s, Out<float> out_hc, In<float> block_out,
+                                            In<float> residual_hc, In<float> split, uint32_t n_w, uint32_t n_embd,
+                                            uint32_t n_hc, uint32_t batch) {
+        return launch_from_split_batched_add2(s, out_hc, block_out, In<float>(), In<float>(), residual_hc, split,
+                                              n_w, n_embd, n_hc, batch);
+    }
+};
+
 // ---- het::dispatch (crates/v4flash-kernels/src/het/dispatch.rs) ------------------------------
 namespace dispatch {
 

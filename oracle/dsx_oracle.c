@@ -486,6 +486,30 @@ void dsx_ref_rms_norm(float *out, const float *x, const float *weight, size_t n,
     }
 }
 
+/* K/kernels/hc_post.hip:15-34 (one token), :40-64 (batched), :66-98 (post / comb from the packed
+ * split row), :100-141 (block = (block_out + add1) + add2).  f32 throughout, the products rounded
+ * before they are added, src ascending. */
+void dsx_ref_hc_post(float *out_hc, const float *block_out, const float *add1, const float *add2,
+                     const float *residual_hc, const float *post, const float *comb, size_t n_embd,
+                     size_t n_hc, size_t b, size_t post_stride, size_t comb_stride) {
+    for (size_t t = 0; t < b; t++) {
+        const float *pb = post + t * post_stride, *cb = comb + t * comb_stride;
+        const float *rh = residual_hc + t * n_hc * n_embd;
+        for (size_t dst = 0; dst < n_hc; dst++)
+            for (size_t d = 0; d < n_embd; d++) {
+                float bv = block_out[t * n_embd + d];
+                if (add1) bv = bv + add1[t * n_embd + d];
+                if (add2) bv = bv + add2[t * n_embd + d];
+                float acc = bv * pb[dst];
+                for (size_t src = 0; src < n_hc; src++) {
+                    const float prod = cb[dst + src * n_hc] * rh[src * n_embd + d];
+                    acc = acc + prod;
+                }
+                out_hc[(t * n_hc + dst) * n_embd + d] = acc;
+            }
+    }
+}
+
 /* ------------------------------------------------------------------------ */
 /* router                                                                    */
 /* ------------------------------------------------------------------------ */

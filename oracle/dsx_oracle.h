@@ -14,6 +14,9 @@
  *   sqrt-softplus / sigmoid routers ................... pinned by f64 ranking
  *   softmax router, group-limited top-k ............... not in the reference;
  *       pinned by brute-force enumeration and numpy primitives
+ *   hc_post (hyper-connection combine) ................ pinned by the f64 closed
+ *       form written out with numpy, an asymmetric mixing matrix (a transposed
+ *       index fails), and the cases that reduce to a copy / a scale
  *   whole-layer composition ........................... pinned by invariants
  *       (token permutation, pick-set split, per-token == batched); end-to-end
  *       agreement with the external ds4 activation dumps is "parity unpinned"
@@ -90,6 +93,12 @@ float dsx_ref_swiglu(float g, float u, float clamp, float ew);
 /* kernels/kernels/rms_norm.hip:12-50 (256 f64 strided partials, f32 tree). */
 void dsx_ref_rms_norm(float *out, const float *x, const float *weight, size_t n, float eps,
                       size_t rows);
+/* kernels/kernels/hc_post.hip:15-34, 40-64, 66-98, 100-141: the hyper-connection combine behind
+ * the FFN, out_hc[t, dst, d] = block[t, d] * post[t, dst] + sum_src comb[t, dst + src * n_hc] *
+ * residual_hc[t, src, d] with block = block_out (+ add1 (+ add2)); add1 / add2 may be NULL. */
+void dsx_ref_hc_post(float *out_hc, const float *block_out, const float *add1, const float *add2,
+                     const float *residual_hc, const float *post, const float *comb, size_t n_embd,
+                     size_t n_hc, size_t b, size_t post_stride, size_t comb_stride);
 
 /* ---- router ---------------------------------------------------------------
  * selected[T,n_used] (int32), weights[T,n_used].  bias may be NULL.  n_group<=1

@@ -116,6 +116,8 @@ def _declare(l):
     l.dsx_ref_swiglu.restype = f32
     l.dsx_ref_swiglu.argtypes = [f32, f32, f32, f32]
     l.dsx_ref_rms_norm.argtypes = [vp, vp, vp, sz, f32, sz]
+    l.dsx_ref_hc_post.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz]
+    l.dsx_ref_hc_post.restype = None
     l.dsx_ref_router_topk.restype = i32
     l.dsx_ref_router_topk.argtypes = [vp, vp, vp, vp, i32, i32, f32, f32, i32, i32, i32, i32]
     l.dsx_ref_router_scores.restype = i32
@@ -279,6 +281,38 @@ def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
     rows, n = x.shape
     out = np.empty_like(x)
     lib().dsx_ref_rms_norm(_p(out), _p(x), _p(weight), n, eps, rows)
+    return out
+
+
+def hc_post(block_out, residual_hc, post, comb, add1=None, add2=None) -> np.ndarray:
+    """crates/v4flash-kernels/kernels/hc_post.hip:15-34,40-64,100-141.  block_out [b, n_embd],
+    residual_hc [b, n_hc, n_embd], post [b, n_hc], comb [b, n_hc, n_hc] addressed
+    [dst + src * n_hc] (so comb[t, src, dst] as a numpy array) -> out_hc [b, n_hc, n_embd]."""
+    block_out, residual_hc = _c(block_out, np.float32), _c(residual_hc, np.float32)
+    post, comb = _c(post, np.float32), _c(comb, np.float32)
+    b, n_hc, n_embd = residual_hc.shape
+    assert block_out.shape == (b, n_embd) and post.shape == (b, n_hc) and comb.shape == (b, n_hc, n_hc)
+    add1 = None if add1 is None else _c(add1, np.float32)
+    add2 = None if add2 is None else _c(add2, np.float32)
+    out = np.empty_like(residual_hc)
+    lib().dsx_ref_hc_post(_p(out), _p(block_out), _p(add1), _p(add2), _p(residual_hc), _p(post),
+                          _p(comb), n_embd, n_hc, b, n_hc, n_hc * n_hc)
+    return out
+
+
+def hc_post_from_split(block_out, residual_hc, split, n_w, add1=None, add2=None) -> np.ndarray:
+    """crates/v4flash-kernels/kernels/hc_post.hip:66-98: post and comb read from the packed row
+    split[b, n_w + n_hc + n_hc * n_hc] (post at n_w, comb behind it)."""
+    block_out, residual_hc, split = _c(block_out, np.float32), _c(residual_hc, np.float32), _c(split, np.float32)
+    b, n_hc, n_embd = residual_hc.shape
+    stride = n_w + n_hc + n_hc * n_hc
+    assert split.shape == (b, stride)
+    add1 = None if add1 is None else _c(add1, np.float32)
+    add2 = None if add2 is None else _c(add2, np.float32)
+    out = np.empty_like(residual_hc)
+    flat = split.reshape(-1)
+    lib().dsx_ref_hc_post(_p(out), _p(block_out), _p(add1), _p(add2), _p(residual_hc),
+                          _p(flat[n_w:]), _p(flat[n_w + n_hc:]), n_embd, n_hc, b, stride, stride)
     return out
 
 

@@ -110,6 +110,9 @@ void host_only_checks() {
            st.message);
     st = dispatch::reduce_partials(s, Out<float>(fake, 100), In<float>(fake, 100), {}, 8, 64, 2);
     expect(!st.ok(), "reduce_partials refuses a short out", st.message);
+    st = HcPost::launch_batched(s, Out<float>(fake, 2 * 4 * 64), In<float>(fake, 2 * 64), In<float>(fake, 2 * 4 * 64),
+                                In<float>(fake, 8), In<float>(fake, 31), 64, 4, 2);
+    expect(!st.ok() && st.message.find("hc_post comb") != std::string::npos, "HcPost refuses a short comb", st.message);
     MoeExecutor none;
     st = none.run(s, Out<float>(fake, 16), In<float>(fake, 16), In<float>(fake, 16), 1);
     expect(!st.ok() && st.message.find("not created") != std::string::npos, "MoeExecutor refuses to run uncreated");
@@ -378,6 +381,51 @@ void gpu_case(const char *name, dsx::GgufType fmt, int hidden, int inter, int E,
 
 }  // namespace
 
+// HcPost (crates/v4flash-kernels/src/head.rs:269-500) through the wrappers, bit for bit against the oracle:
+// separate post / comb arrays, then the same values inside packed split rows with both addends.
+void hc_post_case() {
+    using namespace dsx;
+    const uint32_t b = 3, n_hc = 4, n_embd = 512, n_w = 5, stride = n_w + n_hc + n_hc * n_hc;
+    std::mt19937_64 rng(77);
+    const auto block = normals(rng, (size_t)b * n_embd, 1.0f), a1 = normals(rng, (size_t)b * n_embd, 1.0f);
+    const auto a2 = normals(rng, (size_t)b * n_embd, 1.0f), res = normals(rng, (size_t)b * n_hc * n_embd, 1.0f);
+    const auto split = normals(rng, (size_t)b * stride, 1.0f);
+    std::vector<float> post((size_t)b * n_hc), comb((size_t)b * n_hc * n_hc);
+    for (uint32_t t = 0; t < b; t++) {
+        std::copy_n(&split[(size_t)t * stride + n_w], n_hc, &post[(size_t)t * n_hc]);
+        std::copy_n(&split[(size_t)t * stride + n_w + n_hc], n_hc * n_hc, &comb[(size_t)t * n_hc * n_hc]);
+    }
+    Stream s;
+    if (!must(Stream::create(s), "hc_post stream")) return;
+    DeviceBuffer<float> d_block, d_a1, d_a2, d_res, d_split, d_post, d_comb, d_out;
+    if (!must(DeviceBuffer<float>::from_host(d_block, block), "hc_post upload") ||
+        !must(DeviceBuffer<float>::from_host(d_a1, a1), "hc_post upload") ||
+        !must(DeviceBuffer<float>::from_host(d_a2, a2), "hc_post upload") ||
+        !must(DeviceBuffer<float>::from_host(d_res, res), "hc_post upload") ||
+        !must(DeviceBuffer<float>::from_host(d_split, split), "hc_post upload") ||
+        !must(DeviceBuffer<float>::from_host(d_post, post), "hc_post upload") ||
+        !must(DeviceBuffer<float>::from_host(d_comb, comb), "hc_post upload") ||
+        !must(DeviceBuffer<float>::zeroed(d_out, res.size()), "hc_post out"))
+        return;
+    std::vector<float> got(res.size()), want(res.size());
+    if (!must(HcPost::launch_batched(s, d_out.view(), d_block.view(), d_res.view(), d_post.view(), d_comb.view(),
+                                     n_embd, n_hc, b), "HcPost::launch_batched") ||
+        !must(s.synchronize(), "hc_post sync") || !must(d_out.copy_to_host(got), "hc_post download"))
+        return;
+    dsx_ref_hc_post(want.data(), block.data(), nullptr, nullptr, res.data(), post.data(), comb.data(), n_embd, n_hc,
+                    b, n_hc, n_hc * n_hc);
+    expect(std::memcmp(got.data(), want.data(), got.size() * 4) == 0, "HcPost::launch_batched equals the oracle bit for bit");
+    if (!must(HcPost::launch_from_split_batched_add2(s, d_out.view(), d_block.view(), d_a1.view(), d_a2.view(),
+                                                     d_res.view(), d_split.view(), n_w, n_embd, n_hc, b),
+              "HcPost::launch_from_split_batched_add2") ||
+        !must(s.synchronize(), "hc_post sync") || !must(d_out.copy_to_host(got), "hc_post download"))
+        return;
+    dsx_ref_hc_post(want.data(), block.data(), a1.data(), a2.data(), res.data(), split.data() + n_w,
+                    split.data() + n_w + n_hc, n_embd, n_hc, b, stride, stride);
+    expect(std::memcmp(got.data(), want.data(), got.size() * 4) == 0,
+           "HcPost::launch_from_split_batched_add2 equals the oracle bit for bit");
+}
+
 int main(int argc, char **argv) {
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host-only") == 0;
     host_only_checks();
@@ -395,6 +443,7 @@ int main(int argc, char **argv) {
         gpu_case("q8_0 softmax", dsx::GgufType::Q8_0, 256, 384, 16, 6, 384, 4,
                  {dsx::RouterMode::Softmax, false, 1, 1, 1.0f, 1e-20f}, 0xD5EE0003ull);
     }
+    if (!host_only) hc_post_case();
     std::printf("%s: %d checks, %d failed%s\n", g_failed == 0 ? "PASS" : "FAIL", g_checks, g_failed,
                 host_only ? " (host only)" : "");
     return g_failed == 0 ? 0 : 1;
