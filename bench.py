@@ -36,20 +36,51 @@ DOMINANT_KERNEL = "k_mxfp4_decode_fused<8,false,false>"
 # copy below, whose traffic is known).  The figure is read from the committed summary, which
 # names the kernel it was taken on; a summary for another kernel gives None (not measured).
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "moe_layer_decode_T1_cfg2_hbm_counters.txt")
+# ... and its average duration under `rocprofv3 --kernel-trace` (line `kernel_trace_avg_us <kernel> <us>`)
+TRACE_SUMMARY = os.path.join(ROOT, "profiles", "moe_layer_decode_T1_cfg2_kernel_trace.txt")
+
+
+def kernel_sources_sha16() -> str:
+    """First 16 hex digits of the SHA-256 over the library's kernel sources (csrc/, names and
+    contents in sorted order): the committed summaries carry the value they were taken at."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "deepstrix_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        h.update(name.encode())
+        with open(os.path.join(csrc, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def summary_figure(path: str, key: str, kernel: str):
+    """(value, source) from the line `<key> <kernel> <value>` of a committed profile summary --
+    (None, reason) when there is no such line, or when the summary says (line `sources_sha16 <hash>`)
+    that it was taken on other kernel sources than the ones in this tree."""
+    rel = os.path.relpath(path, ROOT)
+    value, sha = None, None
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.lstrip("# ").split()
+                if len(parts) >= 3 and parts[0] == key and parts[1] == kernel:
+                    value = float(parts[2])
+                if len(parts) >= 2 and parts[0] == "sources_sha16":
+                    sha = parts[1]
+    except OSError:
+        pass
+    if value is None:
+        return None, f"no `{key}` line for {kernel} in {rel}"
+    now = kernel_sources_sha16()
+    if sha != now:
+        return None, f"{rel} was taken on kernel sources {sha}, this tree has {now}: stale, not quoted"
+    return value, rel
 
 
 def measured_traffic(kernel: str):
-    """(bytes per launch, source) from the line `traffic_bytes_per_launch <kernel> <bytes>` of
-    the committed counter summary; (None, reason) when there is none for this kernel."""
-    try:
-        with open(TRAFFIC_SUMMARY) as f:
-            for line in f:
-                parts = line.lstrip("# ").split()
-                if len(parts) >= 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == kernel:
-                    return int(parts[2]), os.path.relpath(TRAFFIC_SUMMARY, ROOT)
-    except OSError:
-        pass
-    return None, f"no counter summary for {kernel} in {os.path.relpath(TRAFFIC_SUMMARY, ROOT)}"
+    """(bytes per launch, source) of the dominant kernel from the committed counter summary."""
+    v, src = summary_figure(TRAFFIC_SUMMARY, "traffic_bytes_per_launch", kernel)
+    return (None if v is None else int(v)), src
 
 
 class Hip:
@@ -235,11 +266,90 @@ def chain_leg(H, torch, np, n_layers=8, T=2, steps=256, planar=False):
     lat_g = timed(chain.replay)
     q = lambda a: {"p10": float(np.percentile(a, 10)), "p50": float(np.percentile(a, 50)),
                    "p90": float(np.percentile(a, 90))}
-    per_step_bytes = n_layers * T * 9 * EXPERT_BYTES
+    # Algorithmic bytes of a step: per block the distinct routed experts of its T tokens plus the
+    # shared expert ONCE (the definition of the decode legs).  The distinct count is measured on
+    # the first steps with the block's operators called one by one (same picks as the fused block).
+    from deepstrix_amd import dispatch
+    distinct, n_probe = [], 16
+    xn = torch.empty((T, hidden), dtype=torch.float32, device="cuda")
+    lg = torch.empty((T, H.CFG2.n_expert), dtype=torch.float32, device="cuda")
+    for i in range(n_probe):
+        h.copy_(inputs[i])
+        per_step = 0
+        for layer in chain.layers:
+            w = layer.w
+            dispatch.rms_norm(xn, h, w.norm_w, hidden, w.norm_eps, T)
+            dispatch.router_logits(lg, w.router_w, xn, w.n_expert, hidden, T)
+            out, sel, _ = layer.run(xn, lg, want_routing=True)
+            h += out
+            per_step += len(np.unique(sel.cpu().numpy()))
+        distinct.append(per_step)
+    d_mean = float(np.mean(distinct))
+    per_step_bytes = (d_mean + n_layers) * EXPERT_BYTES
+    streamed_bytes = n_layers * T * 9 * EXPERT_BYTES   # what the launches stream when no two tokens share a pass
+    p50 = float(np.percentile(lat_g, 50))
     return {"layers": n_layers, "tokens_per_step": T, "steps": steps,
             "eager_us_per_step": q(lat_e), "graph_us_per_step": q(lat_g),
             "launches_per_step": n_layers * 3,
-            "graph_GBps_p50": per_step_bytes / (np.percentile(lat_g, 50) * 1e-6) / 1e9}
+            "distinct_routed_experts_per_step": d_mean,
+            "algorithmic_bytes_per_step": per_step_bytes,
+            "graph_GBps_p50": per_step_bytes / (p50 * 1e-6) / 1e9,
+            "graph_frac_of_hbm_peak_p50": per_step_bytes / (p50 * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "streamed_bytes_per_step_upper": streamed_bytes}
+
+
+def decode_leg(layers_of, H, torch, np, base, T, reps=8):
+    """One layer forward for T tokens of config 2, rotating over independent layers.  Returns
+    us/token, the measured distinct routed experts D(T), the algorithmic bytes (D(T) + 1) x
+    23,396,352 and the rate and fraction of the HBM peak they give."""
+    xs, ls, _ = H.host_inputs(H.Shape(**{**base.__dict__, "seed": base.seed + T}), T)
+    xs, ls = torch.from_numpy(xs).cuda(), torch.from_numpy(ls).cuda()
+    o = torch.empty((T, base.hidden), dtype=torch.float32, device="cuda")
+    L = len(layers_of)
+    _, sel, _ = layers_of[0].run(xs, ls, want_routing=True)
+    d_t = int(len(np.unique(sel.cpu().numpy())))
+    for r in range(2):
+        layers_of[r % L].run(xs, ls, out=o)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for r in range(reps):
+        layers_of[r % L].run(xs, ls, out=o)
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t1) * 1e6 / reps
+    nbytes = (d_t + 1) * EXPERT_BYTES
+    return {"us_per_token": us / T, "us_per_layer": us, "distinct_routed_experts": d_t,
+            "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9,
+            "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+
+
+def stream_read_leg(hip, layers, torch, np, synth, stream, reps=200):
+    """What a plain read reaches on this device: 210,567,168 bytes (the size of a decode step's
+    weights) streamed by the library's read kernel from the gate tensors of the rotating layers,
+    so that the 256 MB memory-side cache serves none of it; HIP events around each launch."""
+    sink = torch.zeros(4 * 8192, dtype=torch.int32, device="cuda")
+    srcs = [lay.w.gate.view(-1)[:TOKEN_BYTES] for lay in layers]
+    rate = lambda t: TOKEN_BYTES / (t * 1e-6) / 1e9
+    by_grid = {}
+    for wgs in (1024, 2048, 4096, 8192):   # 4 .. 32 workgroups per compute unit
+        for r in range(8):
+            synth.read_dev(sink, srcs[r % len(srcs)], wgs)
+        torch.cuda.synchronize()
+        evs = [(hip.event(), hip.event()) for _ in range(reps)]
+        for r, (a, b) in enumerate(evs):
+            hip.l.hipEventRecord(a, stream)
+            synth.read_dev(sink, srcs[r % len(srcs)], wgs)
+            hip.l.hipEventRecord(b, stream)
+        torch.cuda.synchronize()
+        us = np.array([hip.elapsed_ms(a, b) for a, b in evs]) * 1e3
+        by_grid[wgs] = {"us_event_bracket": {"p10": float(np.percentile(us, 10)), "p50": float(np.percentile(us, 50)),
+                                             "p90": float(np.percentile(us, 90))},
+                        "GBps_p50": rate(np.percentile(us, 50)), "GBps_best": rate(us.min())}
+    best = max(by_grid, key=lambda g: by_grid[g]["GBps_p50"])
+    return {"kernel": "k_read16 (libdsx_synth.so): 256 threads per workgroup, four 16-byte loads in flight per thread",
+            "bytes_per_launch": TOKEN_BYTES, "buffers_rotated": len(srcs), "by_workgroups": by_grid,
+            "best_workgroups": best, "us_event_bracket": by_grid[best]["us_event_bracket"],
+            "GBps_p50": by_grid[best]["GBps_p50"], "GBps_best": by_grid[best]["GBps_best"],
+            "frac_of_hbm_peak_p50": by_grid[best]["GBps_p50"] / HBM_PEAK_GBS}
 
 
 def main():
@@ -254,6 +364,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the informative legs: T=4/16/64 of config 2 and configs 5 and 1")
     ap.add_argument("--no-small-t", action="store_true", help="skip only the T=4/16/64 legs")
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip the plain streaming-read leg (what a read of a decode step's size reaches)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -263,7 +375,7 @@ def main():
 
     import numpy as np
     import torch
-    from deepstrix_amd import capi
+    from deepstrix_amd import capi, synth
     from deepstrix_amd.executor import MoeLayer
     from deepstrix_amd import workloads as H
 
@@ -316,6 +428,7 @@ def main():
     gu_avg_us = float(gu_ms.mean() * 1e3)
     achieved = TOKEN_BYTES / (gu_avg_us * 1e-6) / 1e9
     traffic, traffic_source = measured_traffic(DOMINANT_KERNEL)
+    trace_us, trace_source = summary_figure(TRACE_SUMMARY, "kernel_trace_avg_us", DOMINANT_KERNEL)
 
     # what the bracket itself costs: the same pair of events around a one-workgroup kernel
     # (a 16-byte add, about a microsecond of kernel time in a kernel trace)
@@ -340,7 +453,6 @@ def main():
     empty_us = float(np.median([hip.elapsed_ms(a, b) for a, b in empty]) * 1e3)
 
     # a copy of known size, so that byte counters collected over this run can be scaled
-    from deepstrix_amd import synth
     c_src = torch.empty(COPY_BYTES, dtype=torch.uint8, device="cuda").random_(0, 255)
     c_dst = torch.empty_like(c_src)
     for _ in range(4):
@@ -358,19 +470,14 @@ def main():
              "chain_us_p50_events": float(np.median(chain_ms) * 1e3),
              "layer_GBps_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9,
              "layer_frac_of_hbm_peak_T1": TOKEN_BYTES / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    for T in (() if (args.no_extra or args.no_small_t) else (4, 16, 64)):
-        xs, ls, _ = H.host_inputs(H.Shape(**{**base.__dict__, "seed": base.seed + T}), T)
-        xs, ls = torch.from_numpy(xs).cuda(), torch.from_numpy(ls).cuda()
-        o = torch.empty((T, base.hidden), dtype=torch.float32, device="cuda")
-        reps = 8
-        for r in range(2):
-            layers[r % L].run(xs, ls, out=o)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        for r in range(reps):
-            layers[r % L].run(xs, ls, out=o)
-        torch.cuda.synchronize()
-        extra[f"us_per_token_T{T}"] = (time.perf_counter() - t1) * 1e6 / reps / T
+    small_t = () if (args.no_extra or args.no_small_t) else (4, 16, 64)
+    for T in small_t:
+        leg = decode_leg(layers, H, torch, np, base, T)
+        extra[f"us_per_token_T{T}"] = leg["us_per_token"]
+        extra[f"decode_T{T}"] = leg
+
+    if not args.no_ceiling:
+        extra["stream_read_ceiling"] = stream_read_leg(hip, layers, torch, np, synth, stream)
 
     if not args.no_prefill:
         # The figures of the leg are those of the engine's weight rows -- the layout a checkpoint
@@ -398,20 +505,13 @@ def main():
             lps[i % L].run(x_all[i:i + 1], lg_all[i:i + 1], out=out)
         torch.cuda.synchronize()
         extra["us_per_token_T1_planar_weights"] = (time.perf_counter() - t1) * 1e6 / K
-        # ... and the other token counts of config 2 (the grouped GEMMs from 40 tokens on)
-        for T in (() if (args.no_extra or args.no_small_t) else (4, 16, 64)):
-            xs, ls, _ = H.host_inputs(H.Shape(**{**base.__dict__, "seed": base.seed + T}), T)
-            xs, ls = torch.from_numpy(xs).cuda(), torch.from_numpy(ls).cuda()
-            o = torch.empty((T, base.hidden), dtype=torch.float32, device="cuda")
+        # ... and the other token counts of config 2 (the grouped GEMMs from 12 tokens on)
+        for T in small_t:
             lpt = [MoeLayer(lp.w, T) for lp in lps]
-            for r in range(2):
-                lpt[r % L].run(xs, ls, out=o)
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            for r in range(8):
-                lpt[r % L].run(xs, ls, out=o)
-            torch.cuda.synchronize()
-            extra[f"us_per_token_T{T}_planar_weights"] = (time.perf_counter() - t1) * 1e6 / 8 / T
+            leg = decode_leg(lpt, H, torch, np, base, T)
+            extra[f"us_per_token_T{T}_planar_weights"] = leg["us_per_token"]
+            extra[f"decode_T{T}"]["planar_weights"] = {k: leg[k] for k in ("us_per_token", "us_per_layer", "GBps",
+                                                                            "frac_of_hbm_peak")}
             del lpt
         del lps
     if not args.no_chain:
@@ -445,7 +545,17 @@ def main():
                      "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "traffic_source": traffic_source,
-                     "algorithmic_bytes_per_launch": TOKEN_BYTES, "avg_launch_us": gu_avg_us},
+                     "algorithmic_bytes_per_launch": TOKEN_BYTES, "avg_launch_us": gu_avg_us,
+                     # the same fraction from the two clocks there are: `frac` above is the event
+                     # bracket of this run (it includes what the bracket itself costs, see
+                     # extra.event_bracket_of_nothing_us); the kernel-trace figure is the committed
+                     # rocprofv3 summary's average duration of the kernel (None when stale)
+                     "frac_event_bracket": achieved / HBM_PEAK_GBS,
+                     "frac_event_bracket_source": "HIP events on the launch stream around each of this run's "
+                                                  f"{K} launches, mean",
+                     "frac_kernel_trace": (None if trace_us is None
+                                           else TOKEN_BYTES / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBS),
+                     "frac_kernel_trace_source": trace_source, "kernel_trace_avg_us": trace_us},
         "extra": extra,
     }
 

@@ -178,6 +178,31 @@ __global__ __launch_bounds__(256) void k_copy16(uint4 *__restrict__ dst, const u
         dst[i] = src[i];
 }
 
+// Plain streaming read: every thread XORs the 16-byte words it reads (four independent loads per
+// trip) and every wave stores one word of its own (sink holds 4 words per workgroup), so that next
+// to nothing is written back but the loads cannot be dropped.  What a read of a given size reaches on a device: the ceiling a weight-streaming kernel
+// is measured against.
+__global__ __launch_bounds__(256) void k_read16(uint32_t *__restrict__ sink, const uint4 *__restrict__ src,
+                                                uint64_t n16) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    uint4 a = {0u, 0u, 0u, 0u}, b = a, c = a, d = a;
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 3u * stride < n16; i += 4u * stride) {
+        const uint4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2u * stride], v3 = src[i + 3u * stride];
+        a.x ^= v0.x; a.y ^= v0.y; a.z ^= v0.z; a.w ^= v0.w;
+        b.x ^= v1.x; b.y ^= v1.y; b.z ^= v1.z; b.w ^= v1.w;
+        c.x ^= v2.x; c.y ^= v2.y; c.z ^= v2.z; c.w ^= v2.w;
+        d.x ^= v3.x; d.y ^= v3.y; d.z ^= v3.z; d.w ^= v3.w;
+    }
+    for (; i < n16; i += stride) {
+        const uint4 v0 = src[i];
+        a.x ^= v0.x; a.y ^= v0.y; a.z ^= v0.z; a.w ^= v0.w;
+    }
+    uint32_t r = a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    for (int o = 32; o > 0; o >>= 1) r ^= __shfl_xor(r, o, 64);
+    if ((threadIdx.x & 63u) == 0u) sink[blockIdx.x * 4u + (threadIdx.x >> 6)] = r;
+}
+
 }  // namespace
 
 extern "C" {
@@ -240,6 +265,19 @@ int dsx_synth_copy_dev(void *stream, void *dst, const void *src, uint64_t bytes)
     const uint64_t n16 = bytes / 16u;
     const uint32_t grid = (uint32_t)std::min<uint64_t>((n16 + 255) / 256, 256u * 16u);
     hipLaunchKernelGGL(k_copy16, dim3(grid), dim3(256), 0, (hipStream_t)stream, (uint4 *)dst,
+                       (const uint4 *)src, n16);
+    return (int)hipGetLastError();
+}
+
+// Reads `bytes` bytes of src (see k_read16); sink: 4 words per workgroup, i.e. 64 KiB for the
+// default of 4096 workgroups (`workgroups` = 0: sixteen per compute unit of a 256-unit device).
+int dsx_synth_read_dev(void *stream, void *sink, const void *src, uint64_t bytes, uint32_t workgroups) {
+    if (bytes == 0) return 0;
+    if (bytes % 16u || (uintptr_t)src % 16u || (uintptr_t)sink % 4u) return (int)hipErrorInvalidValue;
+    const uint64_t n16 = bytes / 16u;
+    const uint32_t want = workgroups ? workgroups : 256u * 16u;
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((n16 + 255) / 256, want);
+    hipLaunchKernelGGL(k_read16, dim3(grid), dim3(256), 0, (hipStream_t)stream, (uint32_t *)sink,
                        (const uint4 *)src, n16);
     return (int)hipGetLastError();
 }

@@ -41,6 +41,7 @@ def lib() -> C.CDLL:
         l.dsx_synth_mxfp4_dev.argtypes = [vp, vp, u64, u64, u64, u64, u32, f32]
         l.dsx_synth_q8_0_dev.argtypes = [vp, vp, u64, u64, u64, u64, u32, f32]
         l.dsx_synth_copy_dev.argtypes = [vp, vp, vp, u64]
+        l.dsx_synth_read_dev.argtypes = [vp, vp, vp, u64, u32]
         _lib = l
     return _lib
 
@@ -103,3 +104,14 @@ def copy_dev(dst, src) -> None:
                                   src.data_ptr(), src.numel() * src.element_size())
     if rc:
         raise RuntimeError(f"dsx_synth_copy_dev: hip error {rc}")
+
+
+def read_dev(sink, src, workgroups: int = 0) -> None:
+    """Streams `src` through the library's plain read kernel (one word per wave into `sink`, 16 bytes
+    per workgroup): the read rate a device reaches on a buffer of that size."""
+    import torch
+    assert sink.numel() * sink.element_size() >= 16 * (workgroups or 4096)
+    rc = lib().dsx_synth_read_dev(torch.cuda.current_stream().cuda_stream, sink.data_ptr(), src.data_ptr(),
+                                  src.numel() * src.element_size(), workgroups)
+    if rc:
+        raise RuntimeError(f"dsx_synth_read_dev: hip error {rc}")
