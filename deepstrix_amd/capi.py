@@ -95,6 +95,7 @@ SIGNATURES = {
     "dsx_moe_layer_weights_to_rows": (_int, [_vp, _vp]),
     "dsx_moe_layer_set_profile_events": (_int, [_vp, _vp, _vp, _vp]),
     "dsx_moe_layer_set_tuning": (_int, [_vp, _u32, _u32, _u32, _u32]),
+    "dsx_moe_layer_get_tuning": (_int, [_vp, C.POINTER(C.c_uint32 * 6)]),
     "dsx_moe_layer_set_decode": (_int, [_vp, _u32, _u32]),
     "dsx_moe_layer_set_trace": (_int, [_vp, _vp, _sz]),
     "dsx_moe_layer_status": (_int, [_vp, _vp, C.POINTER(C.c_uint32)]),

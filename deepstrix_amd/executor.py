@@ -70,6 +70,13 @@ class LayerWeights:
 
 
 class MoeLayer:
+    # Set by a test-suite whose small shapes stand in for the DeepSeek-V3 shape's paths: layers with
+    # fewer experts than this keep the V3 token thresholds (decode path up to 16 tokens, grouped
+    # GEMM from 100; planar: 11 / 17 / narrow tile below 14 picks), so that a token count names the
+    # same path on them as on the real shape.  None (the default): the library's own,
+    # shape-derived thresholds.
+    v3_thresholds_below_experts: Optional[int] = None
+
     def __init__(self, w: LayerWeights, max_tokens: int):
         capi.init()
         self.w = w
@@ -100,8 +107,18 @@ class MoeLayer:
         h = C.c_void_p()
         check(lib().dsx_moe_layer_create(C.byref(d), C.byref(h)))
         self._h = h
+        self._pin_v3_thresholds()
         self.workspace_bytes = int(lib().dsx_moe_layer_workspace_bytes(h, max_tokens))
         self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=w.gate.device)
+
+    def _pin_v3_thresholds(self):
+        w, lim = self.w, MoeLayer.v3_thresholds_below_experts
+        if lim is None or w.n_expert >= lim:
+            return
+        if w.gate_fmt == FMT_MXFP4_PLANAR and w.down_fmt == FMT_MXFP4_PLANAR:   # (a layer with a Q8_0 matrix keeps the rows' thresholds)
+            self.set_tuning(gemm_min_tokens=17, decode_max_tokens=11, gemm_narrow_members=14)
+        else:
+            self.set_tuning(gemm_min_tokens=100, decode_max_tokens=16, gemm_narrow_members=1)
 
     def __del__(self):
         h = getattr(self, "_h", None)
@@ -120,6 +137,7 @@ class MoeLayer:
         for name in ("gate_fmt", "up_fmt", "down_fmt") + (("sh_gate_fmt", "sh_up_fmt", "sh_down_fmt") if w.sh_inter else ()):
             if getattr(w, name) == FMT_MXFP4:
                 setattr(w, name, FMT_MXFP4_PLANAR)
+        self._pin_v3_thresholds()
 
     def weights_to_rows(self):
         check(lib().dsx_moe_layer_weights_to_rows(self._h, torch.cuda.current_stream().cuda_stream))
@@ -127,6 +145,7 @@ class MoeLayer:
         for name in ("gate_fmt", "up_fmt", "down_fmt") + (("sh_gate_fmt", "sh_up_fmt", "sh_down_fmt") if w.sh_inter else ()):
             if getattr(w, name) == FMT_MXFP4_PLANAR:
                 setattr(w, name, FMT_MXFP4)
+        self._pin_v3_thresholds()
 
     def set_profile_events(self, gate_up_begin=None, gate_up_end=None, down_end=None):
         """hipEvent_t handles (ints) recorded around the gate/up launch and after down."""
@@ -137,6 +156,13 @@ class MoeLayer:
         """0 keeps the current value (include/dsx_moe.h: dsx_moe_layer_set_tuning)."""
         check(lib().dsx_moe_layer_set_tuning(self._h, by_expert_chunk, gemm_min_tokens,
                                              decode_max_tokens, gemm_narrow_members))
+
+    def tuning(self) -> dict:
+        """The thresholds in force (include/dsx_moe.h: dsx_moe_layer_get_tuning)."""
+        v = (C.c_uint32 * 6)()
+        check(lib().dsx_moe_layer_get_tuning(self._h, C.byref(v)))
+        return dict(zip(("by_expert_chunk", "gemm_min_tokens", "gemm_q8_min_tokens", "decode_max_tokens",
+                         "gemm_narrow_members", "share_min_tokens"), (int(x) for x in v)))
 
     def set_decode(self, fused: int = 0, spin_limit: int = 0):
         """fused: 1 = one launch for gate/up + down, pairing tokens that name one expert from 4

@@ -331,23 +331,33 @@ int dsx_moe_layer_weights_to_rows(dsx_moe_layer *layer, dsx_stream_t stream);
  * launch and after the down launch, so a harness can time the dominant kernel in place. */
 int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, void *gate_up_end,
                                      void *down_end);
-/* Tuning knobs with no counterpart in the reference; 0 keeps the current value.
+/* Tuning knobs with no counterpart in the reference; 0 keeps the current value.  The defaults follow
+ * from the layer's shape: which path a token count takes depends on the picks an expert receives,
+ * T * n_used / n_expert (in brackets: the DeepSeek-V3 shape, 256 experts, top-8).
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens (default 100; 17 on planar weights): from this many tokens on, a layer with MXFP4 gate/up runs the
- * grouped-GEMM path (128 token columns per work item, shared expert as an extra group; a Q8_0
- * down matrix takes the int8 grouped GEMM -- layers with a Q8_0 matrix keep 100 on planar weights too);
- * an all-MXFP4 layer whose GEMMs use the narrow tile (below) switches at 11/16 of it.
- * decode_max_tokens (default 16; 11 on planar weights): up to this many tokens, an all-MXFP4 layer runs the decode path
- * (dsx_moe_layer_set_decode: every token on its own picks, no grouping by expert; the one-launch
- * form serves at most 16 tokens, beyond that the decode kernels run once per stage).
- * gemm_narrow_members (default 1 = never; 14 on planar weights): while the picks per expert average less than this,
- * the all-MXFP4 grouped GEMMs use 16 token columns per work item and two workgroups per CU. */
+ * gemm_min_tokens (default: 3.125 picks per expert [100 tokens]; 6.5 for matrices under 4 M elements;
+ * all-Q8_0 layers 1.5; on planar weights right behind the decode path [17]): from this many tokens
+ * on, a layer with MXFP4 gate/up runs the grouped-GEMM path (128 token columns per work item,
+ * shared expert as an extra group; a Q8_0 down matrix takes the int8 grouped GEMM) and an all-Q8_0
+ * layer the int8 grouped GEMMs; an all-MXFP4 layer whose GEMMs use the narrow tile (below)
+ * switches at 11/16 of it.
+ * decode_max_tokens (default: 0.7 picks per expert, at most 16 [16]; 0.375 on planar weights [11]):
+ * up to this many tokens, an all-MXFP4 layer runs the decode path (dsx_moe_layer_set_decode: every
+ * token on its own picks, no grouping by expert; the one-launch form serves at most 16 tokens,
+ * beyond that the decode kernels run once per stage).
+ * gemm_narrow_members (default 1 = never; 14 on planar weights): while the picks per expert average
+ * less than this, the all-MXFP4 grouped GEMMs use 16 token columns per work item and two
+ * workgroups per CU. */
 int dsx_moe_layer_set_tuning(dsx_moe_layer *layer, uint32_t by_expert_chunk, uint32_t gemm_min_tokens,
                              uint32_t decode_max_tokens, uint32_t gemm_narrow_members);
+/* The current values: out[0] by_expert_chunk, [1] gemm_min_tokens, [2] the same for layers whose
+ * GEMMs are int8 (all-Q8_0), [3] decode_max_tokens, [4] gemm_narrow_members, [5] the token count
+ * from which the one-launch decode path pairs tokens that name one expert (0: never). */
+int dsx_moe_layer_get_tuning(const dsx_moe_layer *layer, uint32_t out[6]);
 /* Decode path of an all-MXFP4 layer (up to decode_max_tokens tokens); no counterpart in the
  * reference.  fused: 1 = gate/up, mid quantization, down and the slot-order sum in ONE launch
- * whose workgroups hand results to each other through device memory (the default); from 4
- * tokens on, the tokens of a step that name one expert are paired and the expert is streamed
+ * whose workgroups hand results to each other through device memory (the default); from an eighth
+ * of a pick per expert on (DeepSeek-V3 shape: 4 tokens), the tokens of a step that name one expert are paired and the expert is streamed
  * once per pair (the reference's drafter groups few picks by distinct expert likewise,
  * crates/v4flash-kernels/kernels/mxfp4_pair_matvec.hip:621-782); results are bitwise the same
  * with and without pairing.  3 = the same launch, never pairing; 4 = the same launch, pairing

@@ -43,6 +43,19 @@ def fp8_ue8m0_roundtrip(x: np.ndarray, block: int = 32) -> np.ndarray:
     return (q * s).reshape(x.shape)
 
 
+def int8_pow2_roundtrip(x: np.ndarray, block: int) -> np.ndarray:
+    """x -> dequantized int8 with a POWER-OF-TWO scale per `block` values: s = 2^ceil(log2(amax / 127)),
+    q = rint(x / s) (|q| <= 127 by construction).  The question behind it: such a scale could ride
+    the matrix instruction's E8M0 operand, so that the sums over a row chain through the
+    instruction's accumulator instead of being folded per block on the vector ALU."""
+    x = np.asarray(x, np.float32)
+    g = x.reshape(-1, block).astype(np.float64)
+    amax = np.abs(g).max(axis=1, keepdims=True)
+    s = np.exp2(np.ceil(np.log2(np.maximum(amax, 1e-30) / 127.0)))
+    q = np.clip(np.rint(g / s), -127, 127)
+    return (q * s).reshape(x.shape)
+
+
 def q8k_roundtrip(x: np.ndarray) -> np.ndarray:
     x = np.ascontiguousarray(x, np.float32)
     return ref.q8k_dequant(ref.q8k_quantize(x)).astype(np.float64)
@@ -51,6 +64,8 @@ def q8k_roundtrip(x: np.ndarray) -> np.ndarray:
 ACT_MODES = {
     "q8_k": q8k_roundtrip,                      # the engine's (and this library's) arithmetic
     "fp8_ue8m0_32": fp8_ue8m0_roundtrip,        # one-plane FP8 operand
+    "int8_pow2_256": lambda v: int8_pow2_roundtrip(v, 256),   # int8, power-of-two scale per Q8_K block
+    "int8_pow2_32": lambda v: int8_pow2_roundtrip(v, 32),     # ... per 32 values (the instruction's scale group)
     "none": lambda v: np.asarray(v, np.float64),  # unquantized activations
 }
 
@@ -111,15 +126,20 @@ def compare(a: np.ndarray, b_ref: np.ndarray) -> dict:
 
 
 def study(shape, T: int):
-    """Errors of the one-plane FP8 and of unquantized activations against the Q8_K result, on the
+    """Errors of the one-plane FP8, of int8 with power-of-two scales (per 256 and per 32 values) and
+    of unquantized activations against the Q8_K result, on the
     seeded inputs and GPU-independent oracle routing of `shape` (a tests.helpers.Shape)."""
     from tests import helpers as H
     x, logits, bias = H.host_inputs(shape, T)
     sel, wts = H.oracle_route(shape, logits, bias)
     w = H.host_weights(shape, experts=np.unique(sel))
-    outs = layer_outputs(w, x, sel, wts, ("q8_k", "fp8_ue8m0_32", "none"))
+    outs = layer_outputs(w, x, sel, wts, ("q8_k", "fp8_ue8m0_32", "int8_pow2_256", "int8_pow2_32", "none"))
     return {"fp8_ue8m0_32 vs q8_k": compare(outs["fp8_ue8m0_32"], outs["q8_k"]),
+            "int8_pow2_256 vs q8_k": compare(outs["int8_pow2_256"], outs["q8_k"]),
+            "int8_pow2_32 vs q8_k": compare(outs["int8_pow2_32"], outs["q8_k"]),
             "q8_k vs unquantized": compare(outs["q8_k"], outs["none"]),
+            "int8_pow2_256 vs unquantized": compare(outs["int8_pow2_256"], outs["none"]),
+            "int8_pow2_32 vs unquantized": compare(outs["int8_pow2_32"], outs["none"]),
             "fp8_ue8m0_32 vs unquantized": compare(outs["fp8_ue8m0_32"], outs["none"])}
 
 

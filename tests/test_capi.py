@@ -154,6 +154,47 @@ def test_operators_refuse_bad_arguments_before_any_launch():
     assert l.dsx_last_error()
 
 
+def _thresholds(hidden, inter, n_expert, n_used, gate_fmt=None, down_fmt=None):
+    """Default thresholds of a layer of that shape (no device needed: creating a layer whose
+    shared expert rides with the routed ones only records pointers and sizes)."""
+    import ctypes as C
+    l = capi.lib()
+    d = capi.LayerDesc()
+    d.hidden, d.inter, d.n_expert, d.n_used = hidden, inter, n_expert, n_used
+    d.gate_fmt = d.up_fmt = capi.FMT_MXFP4 if gate_fmt is None else gate_fmt
+    d.down_fmt = capi.FMT_MXFP4 if down_fmt is None else down_fmt
+    d.gate = d.up = d.down = 0x1000
+    d.gate_bpe = d.up_bpe = d.down_bpe = 1 << 20
+    d.router_mode, d.n_group, d.topk_group = 1, 1, 1
+    h = C.c_void_p()
+    assert l.dsx_moe_layer_create(C.byref(d), C.byref(h)) == 0, l.dsx_last_error()
+    v = (C.c_uint32 * 6)()
+    assert l.dsx_moe_layer_get_tuning(h, C.byref(v)) == 0
+    l.dsx_moe_layer_destroy(h)
+    return dict(zip(("chunk", "gemm", "gemm_q8", "decode_max", "narrow", "share"), (int(x) for x in v)))
+
+
+def test_default_thresholds_follow_the_picks_per_expert():
+    """The crossovers measured on four shapes, as picks per expert (include/dsx_moe.h:
+    dsx_moe_layer_set_tuning): the DeepSeek-V3 shape keeps the token counts it was measured at, and
+    other shapes get theirs from the same ratios instead of inheriting V3's token counts."""
+    v3 = _thresholds(7168, 2048, 256, 8)
+    assert (v3["gemm"], v3["decode_max"], v3["narrow"], v3["share"]) == (100, 16, 1, 4)
+    # 128 experts, top-8: by-expert overtakes the decode launch between 12 and 16 tokens, the GEMM
+    # the by-expert kernels between 32 and 48
+    e128 = _thresholds(4096, 1024, 128, 8)
+    assert 11 <= e128["decode_max"] <= 15 and 33 <= e128["gemm"] <= 50
+    # 64 experts, top-6, small matrices: 6 .. 8 tokens and 48 .. 96 tokens
+    e64 = _thresholds(2048, 1536, 64, 6)
+    assert 6 <= e64["decode_max"] <= 7 and 49 <= e64["gemm"] <= 96
+    # config 1 (all Q8_0): the int8 GEMM is ahead from 16 tokens on and far ahead at 24
+    q8 = _thresholds(2048, 1408, 64, 6, capi.FMT_Q8_0, capi.FMT_Q8_0)
+    assert 12 <= q8["gemm_q8"] <= 24
+    # MXFP4 gate/up with a Q8_0 down matrix (config 5) switches with the MXFP4 GEMM
+    mixed = _thresholds(7168, 2048, 256, 8, capi.FMT_MXFP4, capi.FMT_Q8_0)
+    assert mixed["gemm_q8"] == mixed["gemm"] == 100
+
+
 def test_missing_library_is_an_import_error_not_a_fallback(monkeypatch):
     monkeypatch.setattr(capi, "_lib", None)
     monkeypatch.setattr(capi, "LIB_PATH", os.path.join(ROOT, "deepstrix_amd", "lib", "absent.so"))
