@@ -83,10 +83,10 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_gate_up<2, true, false, false>);
         allow_lds(k_mxfp4_gate_up<4, true, false, false>);
         allow_lds(k_mxfp4_gate_up<8, true, false, false>);
-        allow_lds(k_mxfp4_gate_up<1, true, true, false>);
-        allow_lds(k_mxfp4_gate_up<2, true, true, false>);
-        allow_lds(k_mxfp4_gate_up<4, true, true, false>);
-        allow_lds(k_mxfp4_gate_up<8, true, true, false>);
+        allow_lds(k_mxfp4_gate_up_be4<1>);
+        allow_lds(k_mxfp4_gate_up_be4<2>);
+        allow_lds(k_mxfp4_gate_up_be4<4>);
+        allow_lds(k_mxfp4_gate_up_be4<8>);
         allow_lds(k_mxfp4_decode_fused<8, false>);
         allow_lds(k_mxfp4_decode_fused<0, false>);
         allow_lds(k_mxfp4_decode_fused<8, true>);
@@ -113,11 +113,11 @@ void raise_lds_limits() {
         allow_lds(k_mxfp4_down_by_expert<4, false>);
         allow_lds(k_mxfp4_down_by_expert<8, false>);
         allow_lds(k_mxfp4_down_by_expert<16, false>);
-        allow_lds(k_mxfp4_down_by_expert<1, true>);
-        allow_lds(k_mxfp4_down_by_expert<2, true>);
-        allow_lds(k_mxfp4_down_by_expert<4, true>);
-        allow_lds(k_mxfp4_down_by_expert<8, true>);
-        allow_lds(k_mxfp4_down_by_expert<16, true>);
+        allow_lds(k_mxfp4_down_be4<1>);
+        allow_lds(k_mxfp4_down_be4<2>);
+        allow_lds(k_mxfp4_down_be4<4>);
+        allow_lds(k_mxfp4_down_be4<8>);
+        allow_lds(k_mxfp4_down_be4<16>);
         q8_0_raise_lds_limits();
         q8_0_gemm_raise_lds_limits();
     }
@@ -138,8 +138,9 @@ template <int NT>
 static void launch_gate_up_be(hipStream_t st, const GateUpParams &p, uint32_t max_wi, size_t lds,
                               bool staged) {
     const dim3 grid(p.n_rows / 16, max_wi * p.n_sub);
-    if (staged)
-        hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, true, false>), grid, dim3(kGuWaves * 64), lds, st, p);
+    if (staged)   // (four row tiles per workgroup)
+        hipLaunchKernelGGL((k_mxfp4_gate_up_be4<NT>), dim3((p.n_rows / 16 + kGuBeTiles - 1) / kGuBeTiles, grid.y),
+                           dim3(kGuWaves * 64), lds, st, p);
     else
         hipLaunchKernelGGL((k_mxfp4_gate_up<NT, true, false, false>), grid, dim3(kGuWaves * 64), lds, st, p);
 }
@@ -148,8 +149,9 @@ template <int NT>
 static void launch_down_be(hipStream_t st, const DownByExpertParams &p, uint32_t max_wi, size_t lds,
                            bool staged) {
     const dim3 grid(p.n_rows / 16, max_wi * p.n_sub);
-    if (staged)
-        hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, true>), grid, dim3(kDownBeWaves * 64), lds, st, p);
+    if (staged)   // (four row tiles per workgroup)
+        hipLaunchKernelGGL((k_mxfp4_down_be4<NT>), dim3((p.n_rows / 16 + kBe4Waves - 1) / kBe4Waves, grid.y),
+                           dim3(kBe4Waves * 64), lds, st, p);
     else
         hipLaunchKernelGGL((k_mxfp4_down_by_expert<NT, false>), grid, dim3(kDownBeWaves * 64), lds, st, p);
 }
@@ -509,6 +511,8 @@ static int gate_up_be_impl(dsx_stream_t stream, int dtype, float *mid, const uin
     if (n_blocks == 0) return fail(DSX_ERR_INVALID_ARG, "moe_gate_up_chunked_rows: n_blocks=0");
     if (gbpe % 8 || ubpe % 8 || !aligned(gate, 8) || !aligned(up, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: weights must be 8-byte aligned, xq 4-byte");
+    if (staged && !aligned(mid, 16))   // (the staged-row kernels store four rows of a column at a time)
+        return fail(DSX_ERR_SHAPE, "moe_gate_up_chunked_rows: mid must be 16-byte aligned");
     const int nt = fit_nt(chunk, n_blocks, 8);
     const size_t lds = (size_t)n_blocks * 512 * nt + (size_t)n_blocks * nt * 4;
     if (lds > kLdsBudget)
@@ -582,6 +586,8 @@ static int down_be_impl(dsx_stream_t stream, int dtype, float *partials, const u
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: xq_slot_stride=%u", xq_slot_stride);
     if (dbpe % 8 || !aligned(down, 8) || !aligned(xq, staged ? 16 : 4))
         return fail(DSX_ERR_SHAPE, "moe_down_by_expert: weights must be 8-byte aligned, xq 4-byte");
+    if (staged && !aligned(partials, 16))
+        return fail(DSX_ERR_SHAPE, "moe_down_by_expert: partials must be 16-byte aligned");
     const int nt = fit_nt(chunk, n_blocks_in, 16);
     const size_t lds = (size_t)n_blocks_in * 512 * nt + (size_t)n_blocks_in * nt * 4;
     if (lds > kLdsBudget)

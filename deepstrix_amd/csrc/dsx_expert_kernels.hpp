@@ -708,4 +708,254 @@ __global__ __launch_bounds__(kDownBeWaves * 64) void k_mxfp4_down_by_expert(
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// By-expert down and gate/up on staged rows, four row tiles per workgroup.
+// The kernels above give a 16-row tile to a workgroup whose four waves split the k range: every
+// workgroup looks up its item, stages the members' activation rows -- as many bytes as its
+// weights when a few members meet 16 rows of `down` -- and ends in a sum through LDS, for 17 KB
+// (down) or 122 KB (gate/up) of weights.  In the down kernel here wave w owns row tile 4 bx + w
+// over the whole k range, so that one look-up and one staged copy serve four tiles, nothing is
+// exchanged at the end, and four super-blocks of weights are on their way per wave.  The sums keep
+// the association of the kernels above -- super-blocks s = w' (mod 4) in ascending order into
+// accumulator w', then (((0 + a0) + a1) + a2) + a3 -- and so their bits.
+// ---------------------------------------------------------------------------------------
+constexpr int kBe4Waves = 8;    // waves = row tiles of a workgroup of the down kernel
+constexpr int kGuBeTiles = 8;   // row tiles of a workgroup of the gate/up kernel
+
+template <int NT>
+__global__ __launch_bounds__(kBe4Waves * 64) void k_mxfp4_down_be4(const DownByExpertParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ int s_dest[NT];
+
+    const uint32_t nb = p.n_blocks_in;
+    uint8_t *tiles = smem;
+    float *s_yd = (float *)(smem + (size_t)nb * 512u * NT);
+
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t bx = (gridDim.x & 7u) == 0u ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3)
+                                                : blockIdx.x;  // an XCD's row tiles are contiguous
+    const uint32_t row0 = (bx * (uint32_t)kBe4Waves + wave) * 16u;
+    const bool live = row0 < p.n_rows;   // (the last workgroup of a matrix of 16 (4 n + r) rows)
+    const uint32_t n_sub = p.n_sub > 1u ? p.n_sub : 1u;
+    const uint32_t item = blockIdx.y / n_sub;
+    const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;
+    if ((int)item >= *p.n_work_items) return;
+    const uint32_t wi = (uint32_t)p.work_items[item];
+    const uint32_t e = wi >> 16, start = (wi & 0xFFFFu) + col_off;
+    const uint32_t total = (uint32_t)p.group_count[e];
+    if (start >= total) return;  // uniform: this sub-chunk of the item has no members
+    const uint32_t cnt = min(min(p.chunk - col_off, (uint32_t)NT), total - start);
+    const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+    const bool extra = p.sh_down != nullptr && e >= p.n_expert;
+    if (tid < cnt) {
+        const uint32_t m = (uint32_t)p.members[mbase + tid];
+        const uint32_t t = m >> 16, slot = m & 0xFFFFu;
+        s_dest[tid] = (int)(slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot);
+    }
+
+    // the first four super-blocks of the wave's rows go out before the activations are staged
+    // (unconditional: a row shorter than four super-blocks reads its last one again)
+    const uint32_t r = lane & 15u, kb = lane >> 4;
+    const uint32_t wstep = w_step(p.planar != 0u);
+    const WRow wrow = w_row(extra ? p.sh_down : p.down + (uint64_t)e * p.dbpe, (live ? row0 : 0u) + r, nb, p.planar != 0u);
+    const uint32_t last = nb - 1u;
+    WSuper w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        w[i] = load_wsuper(wrow, (uint64_t)min((uint32_t)i, last) * wstep, kb);
+        // (in this order, as the loop below requests them: the compiler's wait for a super-block
+        // is the weaker of what the loop's entry and its back edge allow)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    __syncthreads();
+    stage_copy<NT, kBe4Waves * 64>(tiles, s_yd, cnt, nb, tid,
+                                   StageMembers{p.xq, p.xq_slot_stride, (const uint32_t *)s_dest});
+    __syncthreads();
+    if (!live) return;
+
+    const uint32_t n = lane & 15u;
+    const uint32_t col = (n < cnt) ? n : 0u;
+    v4f acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](uint32_t s, const WSuper &ws, v4f &a) {
+        const BSuper bs = load_bsuper<NT>(tiles + (size_t)s * 512u * NT, kb, col);
+        mfma_super(a, ws, bs, s_yd[s * NT + col], kb);
+    };
+    uint32_t sb = 0;
+    for (; sb + 8u <= nb; sb += 4u) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            compute(sb + (uint32_t)i, w[i], acc[i]);
+            w[i] = load_wsuper(wrow, (uint64_t)(sb + 4u + (uint32_t)i) * wstep, kb);
+            // (each refill stays right behind the products that free its registers: left alone
+            // the compiler multiplies all four super-blocks first and then requests all four)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // up to seven super-blocks are left: those in the registers, then the rest
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (sb + (uint32_t)i < nb) compute(sb + (uint32_t)i, w[i], acc[i]);
+    if (sb + 4u < nb) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (sb + 4u + (uint32_t)i < nb) w[i] = load_wsuper(wrow, (uint64_t)(sb + 4u + (uint32_t)i) * wstep, kb);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (sb + 4u + (uint32_t)i < nb) compute(sb + 4u + (uint32_t)i, w[i], acc[i]);
+    }
+
+    // C layout: the lane holds rows 4 kb + i of the tile for column n
+    float4 o;
+    o.x = ((0.0f + acc[0].x) + acc[1].x + acc[2].x) + acc[3].x;
+    o.y = ((0.0f + acc[0].y) + acc[1].y + acc[2].y) + acc[3].y;
+    o.z = ((0.0f + acc[0].z) + acc[1].z + acc[2].z) + acc[3].z;
+    o.w = ((0.0f + acc[0].w) + acc[1].w + acc[2].w) + acc[3].w;
+    if (n < cnt) *(float4 *)(p.partials + (uint64_t)s_dest[n] * p.n_rows + row0 + kb * 4u) = o;
+}
+
+// gate/up, by expert on staged rows: the workgroup of k_mxfp4_gate_up<NT, true, true, false> -- four
+// waves that split the k range of a 16-row tile and add their sums through LDS -- for kBe4Waves
+// consecutive row tiles, one after the other: one look-up of the item and one staged copy of its
+// members' rows (half as many bytes as a tile's weights at four members) serve all of them, and a
+// tile's first super-blocks are requested before the sums of the tile before it are added up.
+// (A wave per row tile over the whole k range, as in k_mxfp4_down_be4, was 10 % slower here: a wave
+// that walks along a row alone touches every cache line that two of the 136-byte super-blocks
+// share twice, a microsecond apart, where four waves side by side touch it at the same time.)
+template <int NT>
+__global__ __launch_bounds__(kGuWaves * 64) void k_mxfp4_gate_up_be4(const GateUpParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[kGuWaves][2][4][64];
+    __shared__ int s_dest[NT];
+    __shared__ float s_ew[NT];
+    __shared__ uint32_t s_tok[NT];
+
+    const uint32_t nb = p.n_blocks;
+    uint8_t *tiles = smem;
+    float *s_yd = (float *)(smem + (size_t)nb * 512u * NT);
+
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t bx = (gridDim.x & 7u) == 0u ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3)
+                                                : blockIdx.x;
+    const uint32_t tile0 = bx * (uint32_t)kGuBeTiles;
+    const uint32_t n_t = min((uint32_t)kGuBeTiles, p.n_rows / 16u - tile0);   // row tiles of this workgroup
+    const uint32_t n_sub = p.n_sub > 1u ? p.n_sub : 1u;
+    const uint32_t item = blockIdx.y / n_sub;
+    const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;
+    if ((int)item >= *p.n_work_items) return;  // uniform: grid is an upper bound
+    const uint32_t wi = (uint32_t)p.work_items[item];
+    const uint32_t e = wi >> 16, start = (wi & 0xFFFFu) + col_off;
+    const uint32_t total = (uint32_t)p.group_count[e];
+    if (start >= total) return;  // uniform
+    const uint32_t cnt = min(min(p.chunk - col_off, (uint32_t)NT), total - start);
+    const uint32_t mbase = (uint32_t)p.group_offset[e] + start;
+    const bool extra = p.sh_gate != nullptr && e >= p.n_expert;
+    if (tid < cnt) {
+        const uint32_t m = (uint32_t)p.members[mbase + tid];
+        const uint32_t t = m >> 16, slot = m & 0xFFFFu;
+        s_tok[tid] = t;
+        s_dest[tid] = (int)(slot >= p.n_used ? p.n_tokens * p.n_used + t : t * p.n_used + slot);
+        s_ew[tid] = slot >= p.n_used ? 1.0f : p.ew[t * p.n_used + slot];
+    }
+    const float clamp = extra ? p.sh_clamp : p.clamp;
+    const uint8_t *gate_e = extra ? p.sh_gate : p.gate + (uint64_t)e * p.gbpe;
+    const uint8_t *up_e = extra ? p.sh_up : p.up + (uint64_t)e * p.ubpe;
+
+    // the first two super-blocks of a tile (unconditional: a wave without a block of its own reads
+    // the row's last one and never uses it, so that the k loop starts from a known count of loads)
+    const uint32_t r = lane & 15u, kb = lane >> 4;
+    const uint32_t wstep = w_step(p.planar != 0u);
+    WRow grow, urow;
+    WSuper g0, u0, g1, u1;
+    auto first_loads = [&](uint32_t row0) {
+        grow = w_row(gate_e, row0 + r, nb, p.planar != 0u);
+        urow = w_row(up_e, row0 + r, nb, p.planar != 0u);
+        const uint32_t last = nb - 1u;
+        const uint32_t b0 = wave < last ? wave : last, b1 = wave + kGuWaves < last ? wave + kGuWaves : last;
+        g0 = load_wsuper(grow, (uint64_t)(b0) * wstep, kb);
+        u0 = load_wsuper(urow, (uint64_t)(b0) * wstep, kb);
+        g1 = load_wsuper(grow, (uint64_t)(b1) * wstep, kb);
+        u1 = load_wsuper(urow, (uint64_t)(b1) * wstep, kb);
+    };
+    first_loads(tile0 * 16u);
+
+    __syncthreads();  // s_tok visible
+    stage_copy<NT, kGuWaves * 64>(tiles, s_yd, cnt, nb, tid, StageMembers{p.xq, p.xq_row_bytes, s_tok});
+    __syncthreads();
+
+    const uint32_t n = lane & 15u;
+    const uint32_t col = (n < cnt) ? n : 0u;
+    for (uint32_t rt = 0; rt < n_t; rt++) {
+        const uint32_t row0 = (tile0 + rt) * 16u;
+        v4f acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+        auto compute = [&](uint32_t s, const WSuper &g, const WSuper &u) {
+            const BSuper bs = load_bsuper<NT>(tiles + (size_t)s * 512u * NT, kb, col);
+            const float yd = s_yd[s * NT + col];
+            mfma_super(acc_g, g, bs, yd, kb);
+            mfma_super(acc_u, u, bs, yd, kb);
+        };
+        // the k loop of k_mxfp4_gate_up: two super-blocks of weights in flight per matrix, both
+        // refills of an iteration unconditional, each behind the products that free its registers
+#define DSX_AFTER_PRODUCTS() asm volatile("" : "+v"(acc_g), "+v"(acc_u) :: "memory")
+#define DSX_PIN() asm volatile("" ::: "memory")
+        uint32_t sb = wave;
+        while (sb + 3 * kGuWaves < nb) {
+            compute(sb, g0, u0);
+            DSX_AFTER_PRODUCTS();
+            g0 = load_wsuper(grow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
+            u0 = load_wsuper(urow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
+            DSX_PIN();
+            asm volatile("" : "+v"(g1.s.x), "+v"(g1.s.y), "+v"(u1.s.x), "+v"(u1.s.y));
+            compute(sb + kGuWaves, g1, u1);
+            DSX_AFTER_PRODUCTS();
+            g1 = load_wsuper(grow, (uint64_t)((sb + 3 * kGuWaves)) * wstep, kb);
+            u1 = load_wsuper(urow, (uint64_t)((sb + 3 * kGuWaves)) * wstep, kb);
+            DSX_PIN();
+            sb += 2 * kGuWaves;
+        }
+        if (sb < nb) {
+            WSuper g2 = {}, u2 = {};
+            const bool third = sb + 2 * kGuWaves < nb;
+            if (third) {
+                g2 = load_wsuper(grow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
+                u2 = load_wsuper(urow, (uint64_t)((sb + 2 * kGuWaves)) * wstep, kb);
+            }
+            DSX_PIN();
+            compute(sb, g0, u0);
+            if (sb + kGuWaves < nb) compute(sb + kGuWaves, g1, u1);
+            if (third) compute(sb + 2 * kGuWaves, g2, u2);
+        }
+        DSX_AFTER_PRODUCTS();
+#undef DSX_AFTER_PRODUCTS
+#undef DSX_PIN
+        // the next tile's first super-blocks are on their way while this one's sums are added up
+        if (rt + 1u < n_t) first_loads(row0 + 16u);
+
+        // ---- add the waves' partial sums in wave order, SwiGLU, store --------------------
+        s_red[wave][0][0][lane] = acc_g.x;
+        s_red[wave][0][1][lane] = acc_g.y;
+        s_red[wave][0][2][lane] = acc_g.z;
+        s_red[wave][0][3][lane] = acc_g.w;
+        s_red[wave][1][0][lane] = acc_u.x;
+        s_red[wave][1][1][lane] = acc_u.y;
+        s_red[wave][1][2][lane] = acc_u.z;
+        s_red[wave][1][3][lane] = acc_u.w;
+        __syncthreads();
+        if (tid < 16u * cnt) {
+            const uint32_t rr = tid & 15u, j = tid >> 4;
+            const uint32_t l = (rr >> 2) * 16u + j, i = rr & 3u;  // C layout: row 4*(l/16)+i, col l%16
+            float gs = 0.0f, us = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kGuWaves; w++) {
+                gs += s_red[w][0][i][l];
+                us += s_red[w][1][i][l];
+            }
+            p.mid[(uint64_t)s_dest[j] * p.n_rows + row0 + rr] = swiglu_clamp(gs, us, clamp, s_ew[j]);
+        }
+        __syncthreads();   // s_red is written again by the next tile
+    }
+}
+
 }  // namespace dsx

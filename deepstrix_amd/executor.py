@@ -70,11 +70,11 @@ class LayerWeights:
 
 
 class MoeLayer:
-    # Set by a test-suite whose small shapes stand in for the DeepSeek-V3 shape's paths: layers with
-    # fewer experts than this keep the V3 token thresholds (decode path up to 16 tokens, grouped
+    # Set by a test-suite whose small shapes stand in for the paths of a large one: layers with
+    # fewer experts than this get fixed token thresholds (decode path up to 16 tokens, grouped
     # GEMM from 100; planar: 11 / 17 / narrow tile below 14 picks), so that a token count names the
-    # same path on them as on the real shape.  None (the default): the library's own,
-    # shape-derived thresholds.
+    # same path on every small shape.  None (the default): the library's own, shape-derived
+    # thresholds.
     v3_thresholds_below_experts: Optional[int] = None
 
     def __init__(self, w: LayerWeights, max_tokens: int):

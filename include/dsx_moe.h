@@ -335,13 +335,16 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
  * from the layer's shape: which path a token count takes depends on the picks an expert receives,
  * T * n_used / n_expert (in brackets: the DeepSeek-V3 shape, 256 experts, top-8).
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens (default: 3.125 picks per expert [100 tokens]; 6.5 for matrices under 4 M elements;
- * all-Q8_0 layers 1.5; on planar weights right behind the decode path [17]): from this many tokens
+ * gemm_min_tokens (default for an all-MXFP4 layer: 16500 / sqrt(hidden * inter) picks per expert, held
+ * within 3 .. 12 [4.3 picks: 138 tokens]; MXFP4 gate/up with a Q8_0 down matrix 3.125 [100], 6.5 for
+ * matrices under 4 M elements; all-Q8_0 layers 1.5; on planar weights right behind the decode path
+ * [17]): from this many tokens
  * on, a layer with MXFP4 gate/up runs the grouped-GEMM path (128 token columns per work item,
  * shared expert as an extra group; a Q8_0 down matrix takes the int8 grouped GEMM) and an all-Q8_0
  * layer the int8 grouped GEMMs; an all-MXFP4 layer whose GEMMs use the narrow tile (below)
  * switches at 11/16 of it.
- * decode_max_tokens (default: 0.7 picks per expert, at most 16 [16]; 0.375 on planar weights [11]):
+ * decode_max_tokens (default: 0.45 picks per expert -- 0.85 where inter <= 1024 -- and at most 16 [14];
+ * 0.375 on planar weights [11]):
  * up to this many tokens, an all-MXFP4 layer runs the decode path (dsx_moe_layer_set_decode: every
  * token on its own picks, no grouping by expert; the one-launch form serves at most 16 tokens,
  * beyond that the decode kernels run once per stage).

@@ -176,23 +176,25 @@ def _thresholds(hidden, inter, n_expert, n_used, gate_fmt=None, down_fmt=None):
 
 def test_default_thresholds_follow_the_picks_per_expert():
     """The crossovers measured on four shapes, as picks per expert (include/dsx_moe.h:
-    dsx_moe_layer_set_tuning): the DeepSeek-V3 shape keeps the token counts it was measured at, and
-    other shapes get theirs from the same ratios instead of inheriting V3's token counts."""
+    dsx_moe_layer_set_tuning): every shape gets its token counts from the ratios, none inherits the
+    DeepSeek-V3 shape's."""
     v3 = _thresholds(7168, 2048, 256, 8)
-    assert (v3["gemm"], v3["decode_max"], v3["narrow"], v3["share"]) == (100, 16, 1, 4)
-    # 128 experts, top-8: by-expert overtakes the decode launch between 12 and 16 tokens, the GEMM
-    # the by-expert kernels between 32 and 48
+    # by-expert overtakes the decode launch at 13 .. 14 tokens, the GEMM the by-expert kernels at 128 .. 144
+    assert (v3["narrow"], v3["share"]) == (1, 4)
+    assert 13 <= v3["decode_max"] <= 14 and 129 <= v3["gemm"] <= 144
+    # 128 experts, top-8, inter 1024: by-expert overtakes the decode launch between 12 and 16 tokens,
+    # the GEMM the by-expert kernels between 96 and 128
     e128 = _thresholds(4096, 1024, 128, 8)
-    assert 11 <= e128["decode_max"] <= 15 and 33 <= e128["gemm"] <= 50
-    # 64 experts, top-6, small matrices: 6 .. 8 tokens and 48 .. 96 tokens
+    assert 12 <= e128["decode_max"] <= 15 and 97 <= e128["gemm"] <= 129
+    # 64 experts, top-6, small matrices: 4 .. 5 tokens and 96 .. 128 tokens
     e64 = _thresholds(2048, 1536, 64, 6)
-    assert 6 <= e64["decode_max"] <= 7 and 49 <= e64["gemm"] <= 96
+    assert 4 <= e64["decode_max"] <= 5 and 97 <= e64["gemm"] <= 128
     # config 1 (all Q8_0): the int8 GEMM is ahead from 16 tokens on and far ahead at 24
     q8 = _thresholds(2048, 1408, 64, 6, capi.FMT_Q8_0, capi.FMT_Q8_0)
     assert 12 <= q8["gemm_q8"] <= 24
-    # MXFP4 gate/up with a Q8_0 down matrix (config 5) switches with the MXFP4 GEMM
+    # MXFP4 gate/up with a Q8_0 down matrix (config 5): the int8 down GEMM comes earlier
     mixed = _thresholds(7168, 2048, 256, 8, capi.FMT_MXFP4, capi.FMT_Q8_0)
-    assert mixed["gemm_q8"] == mixed["gemm"] == 100
+    assert mixed["gemm_q8"] == 100
 
 
 def test_missing_library_is_an_import_error_not_a_fallback(monkeypatch):
