@@ -115,3 +115,33 @@ def test_config2_v3_shape_decode(T, cfg2_layer):
 def cfg2_layer():
     dw = H.device_weights(H.CFG2)
     return MoeLayer(dw, 64), dw
+
+
+@pytest.mark.parametrize("hidden,inter", [(256, 256), (512, 768), (768, 1280), (1280, 1792), (1792, 512),
+                                          (2304, 2304), (3072, 1024)])
+def test_by_expert_path_over_super_block_counts(hidden, inter):
+    """The by-expert kernels run several row tiles per workgroup and keep four super-blocks of
+    weights in flight (down) or the k range split over the waves (gate/up): rows of 1 .. 12
+    super-blocks cover every way their loops begin and end.  Against the oracle; the first and the
+    last token then run alone on the same picks through the per-stage decode kernels, against the
+    oracle as well."""
+    s = H.Shape(hidden, inter, 8, 3, router_mode=1, route_scale=2.5, clamp=10.0, seed=900 + hidden // 256 + inter)
+    T = 11
+    x, logits, bias = H.host_inputs(s, T)
+    dw = H.device_weights(s)
+    layer = MoeLayer(dw, T)
+    layer.set_tuning(decode_max_tokens=1, gemm_min_tokens=1 << 20)   # by expert at every token count above 1
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    out, sel, w = layer.run(dx, dl, want_routing=True)
+    out = out.clone()
+    torch.cuda.synchronize()
+    sel_h, w_h = sel.cpu().numpy(), w.cpu().numpy()
+    hw = H.host_weights(s, experts=np.unique(sel_h))
+    want = ref.moe_forward(hw, x, sel_h, w_h)
+    H.assert_parity_up_to_rounding_steps(out.cpu().numpy(), want, hw, sel_h, f"{hidden}x{inter}")
+    assert layer.status() == 0
+    layer.set_decode(fused=2)   # one launch per stage: k_mxfp4_gate_up / k_mxfp4_down_decode
+    for t in (0, T - 1):
+        one = layer.run(dx[t:t + 1], None, selected_in=sel[t:t + 1].contiguous(), weights_in=w[t:t + 1].contiguous())
+        torch.cuda.synchronize()
+        assert H.max_rel(one.cpu().numpy(), want[t:t + 1]) < OUT_TOL
