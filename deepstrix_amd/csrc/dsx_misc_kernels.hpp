@@ -580,6 +580,44 @@ __global__ __launch_bounds__(256) void k_q8_0_quantize(int8_t *__restrict__ xq,
 // ---------------------------------------------------------------------------------------
 constexpr int kGbThreads = 1024;
 
+// Exclusive prefix sums of count[0..n) into off[0..n] and of the groups' work items,
+// ceil(count / chunk), into wi_off[0..n] (entry n: the totals), by the first wave of the workgroup:
+// a lane adds up its share of consecutive groups, the lanes scan their sums with shuffles, and
+// every lane writes its groups' offsets (one thread walking 257 groups through LDS took 8 us of the
+// builders' 17).  The caller puts a barrier on either side.
+__device__ __forceinline__ void gb_scan(const int *s_count, int *s_off, int *s_wi_off, uint32_t n,
+                                        uint32_t chunk, uint32_t tid) {
+    if (tid >= 64u) return;
+    const uint32_t per = (n + 63u) / 64u;
+    const uint32_t b = min(n, tid * per), e = min(n, b + per);
+    int sa = 0, sw = 0;
+    for (uint32_t i = b; i < e; i++) {
+        sa += s_count[i];
+        sw += (s_count[i] + (int)chunk - 1) / (int)chunk;
+    }
+    int ia = sa, iw = sw;   // inclusive scan over the lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int ta = __shfl_up(ia, o, 64), tw = __shfl_up(iw, o, 64);
+        if ((int)tid >= o) {
+            ia += ta;
+            iw += tw;
+        }
+    }
+    int ea = ia - sa, ew = iw - sw;
+    for (uint32_t i = b; i < e; i++) {
+        s_off[i] = ea;
+        s_wi_off[i] = ew;
+        ea += s_count[i];
+        ew += (s_count[i] + (int)chunk - 1) / (int)chunk;
+    }
+    if (tid == 63u) {
+        s_off[n] = ia;
+        s_wi_off[n] = iw;
+    }
+}
+
+
 __global__ __launch_bounds__(kGbThreads) void k_group_build(
     int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
     int32_t *__restrict__ members, int32_t *__restrict__ work_items,
@@ -602,20 +640,10 @@ __global__ __launch_bounds__(kGbThreads) void k_group_build(
         if (e >= 0 && (uint32_t)e < n_expert) atomicAdd(&s_count[e], 1);
     }
     __syncthreads();
-    if (tid == 0) {
-        int acc = 0, wacc = 0;
-        for (uint32_t e = 0; e < n_expert; e++) {
-            s_off[e] = acc;
-            s_wi_off[e] = wacc;
-            acc += s_count[e];
-            wacc += (s_count[e] + (int)chunk - 1) / (int)chunk;
-        }
-        s_off[n_expert] = acc;
-        s_wi_off[n_expert] = wacc;
-        // the optional extra group n_expert: every token, slot n_used
-        *n_work_items = wacc + (extra ? (int)((b + chunk - 1) / chunk) : 0);
-    }
+    gb_scan(s_count, s_off, s_wi_off, n_expert, chunk, tid);
     __syncthreads();
+    // the optional extra group n_expert: every token, slot n_used
+    if (tid == 0) *n_work_items = s_wi_off[n_expert] + (extra ? (int)((b + chunk - 1) / chunk) : 0);
     if (extra) {
         const uint32_t base = (uint32_t)s_off[n_expert], wbase = (uint32_t)s_wi_off[n_expert];
         for (uint32_t t = tid; t < b; t += kGbThreads) members[base + t] = (int)((t << 16) | n_used);
@@ -687,19 +715,9 @@ __global__ __launch_bounds__(kGbThreads) void k_group_count(
     for (uint32_t i = 4u * n4 + tid; i < total; i += kGbThreads) count(selected[i]);
     if (extra && tid == 0) s_count[n_expert] = (int)b;
     __syncthreads();
-    if (tid == 0) {
-        int acc = 0, wacc = 0;
-        for (uint32_t e = 0; e < n_groups; e++) {
-            s_off[e] = acc;
-            s_wi_off[e] = wacc;
-            acc += s_count[e];
-            wacc += (s_count[e] + (int)chunk - 1) / (int)chunk;
-        }
-        s_off[n_groups] = acc;
-        s_wi_off[n_groups] = wacc;
-        *n_work_items = wacc;
-    }
+    gb_scan(s_count, s_off, s_wi_off, n_groups, chunk, tid);
     __syncthreads();
+    if (tid == 0) *n_work_items = s_wi_off[n_groups];
     for (uint32_t e = tid; e < n_groups; e += kGbThreads) {
         group_count[e] = s_count[e];
         group_offset[e] = s_off[e];
