@@ -969,8 +969,8 @@ __device__ __forceinline__ void block_sum_256_multi(float (&v)[N], float *red, u
 // One workgroup per expert, up to kRlTokens tokens per pass.  With NORM the row is normalized
 // on the fly: logit = (sum_i w[i] * (x[i] * norm_w[i])) / rms(x) -- the sum of squares and the
 // dot product are accumulated in the same sweep and reduced together, so the kernel has one
-// round of loads on its critical path; the workgroups whose index is a token id then write
-// that token's normalized row.
+// round of loads on its critical path; every workgroup then writes its slice of the tokens'
+// normalized rows.
 // Router weights are f32 or f16 (the engine keeps ffn_gate_inp in f16,
 // crates/v4flash-kernels/src/f16.rs:37-45); products and sums are f32 either way.
 __device__ __forceinline__ float4 router_w4(const float *p) { return *(const float4 *)p; }
@@ -1056,33 +1056,17 @@ __global__ __launch_bounds__(256) void k_router_logits(float *__restrict__ logit
             if ((uint32_t)j < nt) {
                 const float scale = NORM ? 1.0f / sqrtf(red[kRlTokens + j] / (float)hidden + eps) : 1.0f;
                 if (tid == 0) logits[(uint64_t)(t0 + j) * n_expert + e] = red[j] * scale;
-                if (NORM && e == t0 + (uint32_t)j) {
-                    const float *xr = x + (uint64_t)e * hidden;
-                    float *xo = xn + (uint64_t)e * hidden;
-                    for (uint32_t i = tid; i < n4; i += 256u) {
-                        float4 xv = *(const float4 *)(xr + 4u * i);
-                        const float4 nw = *(const float4 *)(norm_w + 4u * i);
-                        xv.x = xv.x * scale * nw.x;
-                        xv.y = xv.y * scale * nw.y;
-                        xv.z = xv.z * scale * nw.z;
-                        xv.w = xv.w * scale * nw.w;
-                        *(float4 *)(xo + 4u * i) = xv;
-                    }
-                    for (uint32_t i = 4u * n4 + tid; i < hidden; i += 256u)
-                        xo[i] = xr[i] * scale * norm_w[i];
+                if (NORM) {
+                    // every workgroup holds every token's scale (the same sums in the same order), so
+                    // each writes its slice of every normalized row, whatever the number of tokens
+                    const uint32_t t = t0 + (uint32_t)j;
+                    const uint32_t lo = (uint32_t)((uint64_t)e * hidden / n_expert);
+                    const uint32_t hi = (uint32_t)((uint64_t)(e + 1u) * hidden / n_expert);
+                    const float *xr = x + (uint64_t)t * hidden;
+                    float *xo = xn + (uint64_t)t * hidden;
+                    for (uint32_t i = lo + tid; i < hi; i += 256u) xo[i] = xr[i] * scale * norm_w[i];
                 }
             }
-        }
-    }
-    // normalized rows whose index has no workgroup (n_tokens > n_expert): workgroup 0 writes them
-    if (NORM && e == 0 && n_tokens > n_expert) {
-        for (uint32_t t = n_expert; t < n_tokens; t++) {
-            const float *xr = x + (uint64_t)t * hidden;
-            double partial = 0.0;
-            for (uint32_t i = tid; i < hidden; i += 256u) partial += (double)xr[i] * xr[i];
-            const float ss = block_sum_256((float)partial, s_red, tid);
-            const float sc = 1.0f / sqrtf(ss / (float)hidden + eps);
-            for (uint32_t i = tid; i < hidden; i += 256u) xn[(uint64_t)t * hidden + i] = xr[i] * sc * norm_w[i];
         }
     }
 }
