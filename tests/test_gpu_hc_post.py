@@ -98,13 +98,13 @@ def test_layer_forward_hc_is_the_operator_on_the_layers_own_output(T):
         _layer_case(SMALL, layer, T)
 
 
-@pytest.mark.parametrize("T", [1, 3, 5, 40, 130])
+@pytest.mark.parametrize("T", [1, 3, 6, 8, 40, 130])
 def test_layer_forward_hc_with_a_shared_expert_of_another_format(T):
-    """The shared expert inside the launch (up to 3 tokens), on the side stream behind a join (5),
+    """The shared expert inside the launch (up to 6 tokens), on the side stream behind a join (8),
     and beside the by-expert / GEMM paths."""
     layer = MoeLayer(H.device_weights(SMALL_Q8_SHARED), T)
     _layer_case(SMALL_Q8_SHARED, layer, T)
-    if T <= 5:
+    if T <= 8:
         layer.set_decode(fused=2)
         _layer_case(SMALL_Q8_SHARED, layer, T)
 

@@ -47,7 +47,7 @@ def _check(s, layer, hw, T, modes=(1,)):
         assert H.compare_stats(out, want)["max_over_max"] < REGRESSION, (T, mode)
 
 
-@pytest.mark.parametrize("T", [1, 2, 3, 5, 14, 16, 64, 130, 300])
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 6, 7, 9, 14, 16, 64, 130, 300])
 def test_small_layer_with_q8_0_shared_expert_of_another_width(T):
     dw = H.device_weights(SMALL)
     layer = MoeLayer(dw, T)
@@ -55,7 +55,7 @@ def test_small_layer_with_q8_0_shared_expert_of_another_width(T):
 
 
 def test_small_layer_pre_norm_block_with_q8_0_shared_expert():
-    """h += layer(RMSNorm(h)) with the residual folded into the one-launch decode path (up to three
+    """h += layer(RMSNorm(h)) with the residual folded into the one-launch decode path (up to six
     tokens: the shared expert inside the launch; more: on the side stream, its rows and the
     residual added behind the join while the launch writes to a row buffer of the workspace)."""
     s = SMALL
@@ -90,11 +90,11 @@ def test_v3_shape_with_q8_0_shared_expert(T, v3_layer):
 
 @pytest.mark.parametrize("T", [2, 4, 12, 24, 130])
 def test_side_stream_shared_expert_under_graph_capture(T, v3_layer):
-    """From four tokens on (decode, by-expert and GEMM paths alike) the Q8_0 shared expert is
+    """From seven tokens on (decode, by-expert and GEMM paths alike) the Q8_0 shared expert is
     computed on a stream of its own, forked from and joined to the caller's: a capture of the
     caller's stream must record both branches, and every replay must give what the eager call
     gives -- bitwise, with the program's own work and synchronizations between the replays.
-    (Two tokens: the shared expert inside the decode launch, no second stream.)"""
+    (Two and four tokens: the shared expert inside the decode launch, no second stream.)"""
     s = V3
     layer, hw = v3_layer
     layer.set_decode(fused=1)
