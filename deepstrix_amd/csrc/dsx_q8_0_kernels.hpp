@@ -47,6 +47,8 @@ struct Q8Params {
     uint32_t n_expert, n_tokens;
     // by-expert: workgroups along grid.y per work item, NT columns each (0 is read as 1)
     uint32_t n_sub;
+    // down, by-expert: consecutive 16-row tiles per workgroup (0 is read as 1)
+    uint32_t row_tiles;
 };
 
 // The lane's share of `rows[r] . x[c]` for R weight rows and NT columns, over all of its blocks.  The
@@ -251,7 +253,8 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_by_expert(const Q8P
     __shared__ uint32_t s_dest[NT];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t n_sub = p.n_sub > 1u ? p.n_sub : 1u;
-    const uint32_t row0 = blockIdx.x * kQ8RowsPerWg, item = blockIdx.y / n_sub;
+    const uint32_t row_tiles = p.row_tiles > 1u ? p.row_tiles : 1u;
+    const uint32_t row00 = blockIdx.x * row_tiles * kQ8RowsPerWg, item = blockIdx.y / n_sub;
     const uint32_t col_off = (blockIdx.y - item * n_sub) * (uint32_t)NT;
     const uint32_t row_bytes = q8_0_act_row_bytes(p.n_blocks);
     if ((int)item >= *p.n_work_items) return;
@@ -272,24 +275,29 @@ __global__ __launch_bounds__(kQ8Waves * 64) void k_q8_0_down_by_expert(const Q8P
     __syncthreads();
     const uint8_t *w_e = (p.sh_w0 != nullptr && e >= p.n_expert) ? p.sh_w0 : p.w0 + (uint64_t)e * p.bpe0;
     const uint64_t wstride = (uint64_t)p.n_blocks * 34u;
-    // the wave's four rows (wave, wave + 4, ...) at once
-    const uint8_t *base = w_e + (uint64_t)(row0 + wave) * wstride;
-    const uint8_t *const rows[4] = {base, base + kQ8Waves * wstride, base + 2u * kQ8Waves * wstride,
-                                    base + 3u * kQ8Waves * wstride};
-    float a[4][NT];
+    // One look-up of the item and one staged copy of its members' rows serve several row tiles (a
+    // tile's weights are no more bytes than the staged rows of a few members).
+    for (uint32_t rt = 0; rt < row_tiles && row00 + rt * kQ8RowsPerWg < p.n_rows; rt++) {
+        const uint32_t row0 = row00 + rt * kQ8RowsPerWg;
+        // the wave's four rows (wave, wave + 4, ...) at once
+        const uint8_t *base = w_e + (uint64_t)(row0 + wave) * wstride;
+        const uint8_t *const rows[4] = {base, base + kQ8Waves * wstride, base + 2u * kQ8Waves * wstride,
+                                        base + 3u * kQ8Waves * wstride};
+        float a[4][NT];
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+        for (int r = 0; r < 4; r++)
 #pragma unroll
-        for (int c = 0; c < NT; c++) a[r][c] = 0.0f;
-    q8_0_rows_partial<4, NT>(a, rows, lds_x, row_bytes, p.n_blocks, lane);
+            for (int c = 0; c < NT; c++) a[r][c] = 0.0f;
+        q8_0_rows_partial<4, NT>(a, rows, lds_x, row_bytes, p.n_blocks, lane);
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+        for (int r = 0; r < 4; r++)
 #pragma unroll
-        for (int c = 0; c < NT; c++) {
-            const float v = wave_sum_f32(a[r][c]);
-            if (lane == 0 && (uint32_t)c < cnt)
-                p.dst[(uint64_t)s_dest[c] * p.n_rows + row0 + wave + (uint32_t)r * kQ8Waves] = v;
-        }
+            for (int c = 0; c < NT; c++) {
+                const float v = wave_sum_f32(a[r][c]);
+                if (lane == 0 && (uint32_t)c < cnt)
+                    p.dst[(uint64_t)s_dest[c] * p.n_rows + row0 + wave + (uint32_t)r * kQ8Waves] = v;
+            }
+    }
 }
 
 // ---- host side ----------------------------------------------------------------------------
@@ -426,7 +434,13 @@ inline int q8_0_down_by_expert(hipStream_t st, float *partials, const uint8_t *d
     p.n_blocks = n_blocks_in;
     p.sh_w0 = sh_down; p.n_expert = n_expert; p.n_tokens = n_tokens;
     p.n_sub = n_sub;
-    const dim3 grid(n_rows / kQ8RowsPerWg, max_wi * n_sub), block(kQ8Waves * 64);
+    // Two row tiles per workgroup where that still leaves thousands of workgroups: the look-up and the
+    // staged copy then cost half as much per tile (7168 x 2048 down matrices of 256 experts, 24 / 64
+    // tokens: 476 -> 440 / 843 -> 778 us); a small grid needs every workgroup it has (2048 x 1408, 64
+    // experts, 4 tokens: 27 -> 30 us with two tiles).
+    const uint32_t n_tiles = n_rows / kQ8RowsPerWg;
+    p.row_tiles = (uint64_t)n_tiles * max_wi * n_sub >= 16384u ? 2u : 1u;
+    const dim3 grid((n_tiles + p.row_tiles - 1u) / p.row_tiles, max_wi * n_sub), block(kQ8Waves * 64);
     const size_t lds = (size_t)nt * q8_0_act_row_bytes(n_blocks_in);
     switch (nt) {
         case 1: hipLaunchKernelGGL(k_q8_0_down_by_expert<1>, grid, block, lds, st, p); break;
