@@ -145,3 +145,28 @@ def test_by_expert_path_over_super_block_counts(hidden, inter):
         one = layer.run(dx[t:t + 1], None, selected_in=sel[t:t + 1].contiguous(), weights_in=w[t:t + 1].contiguous())
         torch.cuda.synchronize()
         assert H.max_rel(one.cpu().numpy(), want[t:t + 1]) < OUT_TOL
+
+
+def test_by_expert_chunk_sizes_give_the_same_bits():
+    """The members of an expert are served in chunks of `by_expert_chunk` token columns (1 .. 16; the
+    kernels are instantiated for 1, 2, 4, 8 and 16 columns, and a chunk wider than a workgroup's
+    columns is split over several workgroups): every column is computed on its own, so the chunk
+    size must not change a bit of the output."""
+    s = H.Shape(1024, 512, 8, 3, router_mode=1, route_scale=2.5, clamp=10.0, seed=931)
+    T = 40   # 15 picks per expert: several chunks per group at every size
+    x, logits, bias = H.host_inputs(s, T)
+    layer = MoeLayer(H.device_weights(s), T)
+    layer.set_tuning(decode_max_tokens=1, gemm_min_tokens=1 << 20)
+    dx, dl = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    ref_out, sel, w = layer.run(dx, dl, want_routing=True)
+    ref_out = ref_out.clone()
+    sel_h, w_h = sel.cpu().numpy(), w.cpu().numpy()
+    hw = H.host_weights(s, experts=np.unique(sel_h))
+    H.assert_parity_up_to_rounding_steps(ref_out.cpu().numpy(), ref.moe_forward(hw, x, sel_h, w_h), hw, sel_h, "chunk 4")
+    for chunk in (1, 2, 3, 8, 11, 16):
+        layer.set_tuning(by_expert_chunk=chunk)
+        assert layer.tuning()["by_expert_chunk"] == chunk
+        out = layer.run(dx, dl)
+        torch.cuda.synchronize()
+        assert layer.status() == 0
+        assert torch.equal(out, ref_out), f"chunk {chunk}"
