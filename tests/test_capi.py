@@ -192,9 +192,9 @@ def test_default_thresholds_follow_the_picks_per_expert():
     # config 1 (all Q8_0): the int8 GEMM is ahead from 16 tokens on and far ahead at 24
     q8 = _thresholds(2048, 1408, 64, 6, capi.FMT_Q8_0, capi.FMT_Q8_0)
     assert 12 <= q8["gemm_q8"] <= 24
-    # MXFP4 gate/up with a Q8_0 down matrix (config 5): the int8 down GEMM comes earlier
+    # MXFP4 gate/up with a Q8_0 down matrix (config 5): the GEMMs are ahead from 64 tokens on
     mixed = _thresholds(7168, 2048, 256, 8, capi.FMT_MXFP4, capi.FMT_Q8_0)
-    assert mixed["gemm_q8"] == 100
+    assert 49 <= mixed["gemm_q8"] <= 64
 
 
 def test_missing_library_is_an_import_error_not_a_fallback(monkeypatch):
