@@ -196,11 +196,11 @@ int launch_gemm(hipStream_t st, const GemmParams &p, uint32_t max_wi, bool plana
         return fail(DSX_ERR_INVALID_ARG, "gemm: a weight matrix or the activation rows exceed 4 GiB");
     if (planar) {
         hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT, true>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
-                           gemm_lds_bytes(MT), st, p);
+                           gemm_lds_bytes(MT, true), st, p);
         return launched(PAIR ? "gate_up gemm" : "down gemm");
     }
     hipLaunchKernelGGL((k_mxfp4_gemm<PAIR, MT>), dim3((uint32_t)grid), dim3(kGemmWaves * 64),
-                       gemm_lds_bytes(MT), st, p);
+                       gemm_lds_bytes(MT, false), st, p);
     return launched(PAIR ? "gate_up gemm" : "down gemm");
 }
 

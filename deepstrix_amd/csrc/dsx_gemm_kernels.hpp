@@ -41,6 +41,10 @@ constexpr int kGemmRF = 2;                  // 16-row fragments per wave and row
 constexpr int kGemmMT = 128;                // token columns per workgroup (the wide tile)
 constexpr int kGemmMTNarrow = 16;           // ... of the narrow tile: groups of a few members
 constexpr int kGemmAWaveBytes = 2 * kGemmRF * 2048 + 2 * 256;  // a wave's weights of one super-block
+// ... of the wide tile on the engine's rows, which fetches every row's 136 bytes as one run of nine
+// 16-byte pieces (below): two row sets x 5 loads of 1 KB
+constexpr int kGemmARunWaveBytes = 2 * 5 * 1024;
+constexpr int gemm_a_wave_bytes(int mt, bool planar) { return mt == kGemmMT && !planar ? kGemmARunWaveBytes : kGemmAWaveBytes; }
 // LDS of a workgroup.
 // Narrow tile (MT = 16): the operand heads of two half super-blocks of the columns (128 bytes per
 // column each) | the operand tails of two super-blocks (128 bytes per column each: both halves,
@@ -58,7 +62,7 @@ constexpr int gemm_tails_bytes(int mt) { return mt * 128; }
 constexpr int gemm_yd_off(int mt) { return mt == kGemmMT ? 2 * kGemmPhaseBytes : gemm_tails_off(mt) + 2 * gemm_tails_bytes(mt); }
 constexpr int gemm_yd_bytes(int mt) { return mt > 64 ? 2048 : 1024; }
 constexpr int gemm_a_off(int mt) { return gemm_yd_off(mt) + 2 * gemm_yd_bytes(mt); }
-constexpr size_t gemm_lds_bytes(int mt) { return (size_t)gemm_a_off(mt) + kGemmWaves * kGemmAWaveBytes; }
+constexpr size_t gemm_lds_bytes(int mt, bool planar) { return (size_t)gemm_a_off(mt) + kGemmWaves * gemm_a_wave_bytes(mt, planar); }
 
 // f(integral_constant<int, I>) for I = From .. To - 1, unrolled at compile time (the matrix
 // instruction wants its format and scale-select arguments as constants)
@@ -168,8 +172,22 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     static_assert(kGemmRF == 2, "one scale instruction covers the 32 rows of a wave's row set");
     constexpr uint32_t kScaleOff = 2u * kGemmRF * 2048u;
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmAOff + wave * kGemmAWaveBytes);
-    const uint8_t *a_ptr = smem + kGemmAOff + wave * kGemmAWaveBytes;
+    // Wide tile on the engine's rows: a row's super-block -- 128 bytes of nibbles and the 8 scale
+    // bytes behind them -- is fetched as one run of nine 16-byte pieces (the ninth holds bytes
+    // 120..135, so that nothing past the super-block is read), lane slot s = 9 row + piece over the
+    // wave's 32 rows of a row set: 288 slots in five loads.  A run lies in two cache lines, where
+    // the 128-byte piece and the scales on their own made three requests.
+    constexpr bool kRun = MT == kGemmMT && !PLANAR;
+    constexpr int kAWaveBytes = gemm_a_wave_bytes(MT, PLANAR);
+    const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + kGemmAOff + wave * kAWaveBytes);
+    const uint8_t *a_ptr = smem + kGemmAOff + wave * kAWaveBytes;
+    uint32_t run_off[5];   // the lane's byte offset from the first row of the wave's rows, per load of a row set
+#pragma unroll
+    for (int i = 0; i < 5; i++) {
+        const uint32_t slot = min(64u * (uint32_t)i + lane, 287u);   // (the last load's upper half repeats the last piece)
+        const uint32_t rw = (slot * 7282u) >> 16, piece = slot - rw * 9u;   // slot / 9, slot % 9
+        run_off[i] = rw * (p.n_sb * (uint32_t)kSuperBytes) + (piece < 8u ? piece * 16u : 120u);
+    }
     const uint32_t l8 = lane >> 3, c8 = (lane & 7u) ^ l8;
     // fetch side: lane -> row l8 of the 8-row slab, chunk c8
     const uint32_t a_fetch = l8 * row_stride + c8 * 16u;
@@ -186,6 +204,14 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // The part of an address that all lanes share (row set, fragment, super-block) goes into the
     // scalar base of the load; the lane's own offset is the same register for every weight load.
     auto issue_a = [&](uint32_t sb) {
+        if constexpr (kRun) {
+#pragma unroll
+            for (int m = 0; m < 2; m++)
+#pragma unroll
+                for (int i = 0; i < 5; i++)
+                    lds_dma16(a_lds + (uint32_t)(m * 5120 + i * 1024), wbase[m] + (a_slab[0][m] + sb * kStepW), run_off[i]);
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
@@ -228,8 +254,12 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
     // super-block, shared, double buffered; wave w fetches columns 16 w .. 16 w + 15.
     constexpr int kALoads = 4 * kGemmRF + 2;  // per wave and super-block
     // load L of those: 0..7 the halves of the four fragments, 8 and 9 the scales of the row sets
+    // (row runs: loads 0..4 the first row set, 5..9 the second)
     auto issue_a_one = [&](int L, uint32_t sb) __attribute__((always_inline)) {
-        if (L < 4 * kGemmRF) {
+        if constexpr (kRun) {
+            const int m = L / 5, i = L - 5 * m;
+            lds_dma16(a_lds + (uint32_t)(m * 5120 + i * 1024), wbase[m] + (a_slab[0][m] + sb * kStepW), run_off[i]);
+        } else if (L < 4 * kGemmRF) {
             const int f = L >> 1, i = L & 1, r = f >> 1, m = f & 1;
             lds_dma16(a_lds + (uint32_t)(f * 2048 + i * 1024),
                       wbase[m] + (a_slab[r][m] + (uint32_t)i * 8u * row_stride + sb * kStepW), a_fetch);
@@ -255,10 +285,19 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
             for (int m = 0; m < 2; m++) {
-                const uint8_t *f = a_ptr + (r * 2 + m) * 2048;
-                a_cur[r][m].a0 = *(const uint4 *)(f + a_rd);
-                a_cur[r][m].a1 = *(const uint4 *)(f + (a_rd ^ 64u));
-                const uint2 sv = *(const uint2 *)(a_ptr + kScaleOff + m * 256u + r * 128u + n16 * 8u);
+                uint2 sv;
+                if constexpr (kRun) {
+                    // row 16 r + n16 of the row set: pieces g4 and 4 + g4, the scales in the ninth piece's upper half
+                    const uint8_t *f = a_ptr + m * 5120 + ((uint32_t)r * 16u + n16) * 144u;
+                    a_cur[r][m].a0 = *(const uint4 *)(f + g4 * 16u);
+                    a_cur[r][m].a1 = *(const uint4 *)(f + 64u + g4 * 16u);
+                    sv = *(const uint2 *)(f + 136u);
+                } else {
+                    const uint8_t *f = a_ptr + (r * 2 + m) * 2048;
+                    a_cur[r][m].a0 = *(const uint4 *)(f + a_rd);
+                    a_cur[r][m].a1 = *(const uint4 *)(f + (a_rd ^ 64u));
+                    sv = *(const uint2 *)(a_ptr + kScaleOff + m * 256u + r * 128u + n16 * 8u);
+                }
                 a_cur[r][m].sc = ((sv.x >> (g4 * 8u)) & 0xFFu) | (((sv.y >> (g4 * 8u)) & 0xFFu) << 8);
             }
     };
