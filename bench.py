@@ -322,7 +322,7 @@ def decode_leg(layers_of, H, torch, np, base, T, reps=8):
             "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
 
-def stream_read_leg(hip, layers, torch, np, synth, stream, reps=200):
+def stream_read_leg(hip, layers, torch, np, synth, stream, H, reps=200):
     """What a plain read reaches on this device: 210,567,168 bytes (the size of a decode step's
     weights) streamed by the library's read kernel from the gate tensors of the rotating layers,
     so that the 256 MB memory-side cache serves none of it; HIP events around each launch."""
@@ -345,7 +345,32 @@ def stream_read_leg(hip, layers, torch, np, synth, stream, reps=200):
                                              "p90": float(np.percentile(us, 90))},
                         "GBps_p50": rate(np.percentile(us, 50)), "GBps_best": rate(us.min())}
     best = max(by_grid, key=lambda g: by_grid[g]["GBps_p50"])
-    return {"kernel": "k_read16 (libdsx_synth.so): 256 threads per workgroup, four 16-byte loads in flight per thread",
+    # the same bytes read the way the decode kernels stream weights: 16-row tiles of rows of 28
+    # super-blocks (a gate or up matrix of the layer), operand order and memory order
+    n_sb = H.CFG2.hidden // 256
+    n_tiles = TOKEN_BYTES // (16 * n_sb * 136)
+    tile_bytes = n_tiles * 16 * n_sb * 136
+    tiles = {}
+    for name, operand in (("operand_order", True), ("memory_order", False)):
+        for r in range(8):
+            synth.read_tiles_dev(sink, srcs[r % len(srcs)], n_tiles, n_sb, operand)
+        torch.cuda.synchronize()
+        evs = [(hip.event(), hip.event()) for _ in range(reps)]
+        for r, (a, b) in enumerate(evs):
+            hip.l.hipEventRecord(a, stream)
+            synth.read_tiles_dev(sink, srcs[r % len(srcs)], n_tiles, n_sb, operand)
+            hip.l.hipEventRecord(b, stream)
+        torch.cuda.synchronize()
+        us = np.array([hip.elapsed_ms(a, b) for a, b in evs]) * 1e3
+        tiles[name] = {"us_event_bracket": {"p10": float(np.percentile(us, 10)), "p50": float(np.percentile(us, 50)),
+                                            "p90": float(np.percentile(us, 90))},
+                       "GBps_p50": tile_bytes / (np.percentile(us, 50) * 1e-6) / 1e9,
+                       "GBps_best": tile_bytes / (us.min() * 1e-6) / 1e9}
+    return {"weight_tile_pattern": {"kernel": "k_read_tiles (libdsx_synth.so): one workgroup per 16-row tile of 136-byte "
+                                              "super-blocks, four waves on every fourth super-block, two in flight per wave: "
+                                              "the decode kernels' weight loads and nothing else",
+                                    "bytes_per_launch": tile_bytes, **tiles},
+            "kernel": "k_read16 (libdsx_synth.so): 256 threads per workgroup, four 16-byte loads in flight per thread",
             "bytes_per_launch": TOKEN_BYTES, "buffers_rotated": len(srcs), "by_workgroups": by_grid,
             "best_workgroups": best, "us_event_bracket": by_grid[best]["us_event_bracket"],
             "GBps_p50": by_grid[best]["GBps_p50"], "GBps_best": by_grid[best]["GBps_best"],
@@ -477,7 +502,7 @@ def main():
         extra[f"decode_T{T}"] = leg
 
     if not args.no_ceiling:
-        extra["stream_read_ceiling"] = stream_read_leg(hip, layers, torch, np, synth, stream)
+        extra["stream_read_ceiling"] = stream_read_leg(hip, layers, torch, np, synth, stream, H)
 
     if not args.no_prefill:
         # The figures of the leg are those of the engine's weight rows -- the layout a checkpoint

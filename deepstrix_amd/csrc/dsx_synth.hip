@@ -203,6 +203,73 @@ __global__ __launch_bounds__(256) void k_read16(uint32_t *__restrict__ sink, con
     if ((threadIdx.x & 63u) == 0u) sink[blockIdx.x * 4u + (threadIdx.x >> 6)] = r;
 }
 
+
+// The same read, shaped like the decode kernels' weight stream: a matrix of MXFP4 rows (n_sb
+// super-blocks of 136 bytes each), one workgroup per 16-row tile, its four waves taking every fourth
+// super-block, two super-blocks in flight per wave.  OPERAND: every lane loads what the matrix
+// instruction wants from it -- row lane % 16, block lane / 16: 16 bytes at 16 (lane / 16), 16 bytes
+// 64 further on, the row's 8 scale bytes -- as the decode and by-expert kernels do; otherwise the
+// same bytes in memory order (8 rows x 128 bytes per load, the scales by 16 lanes).  What a kernel
+// that reads weights tile by tile reaches, whatever it computes.
+typedef uint32_t rt_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t rt_u32x2 __attribute__((ext_vector_type(2)));
+typedef rt_u32x4 rt_u32x4_a8 __attribute__((aligned(8)));
+typedef rt_u32x2 rt_u32x2_a4 __attribute__((aligned(4)));
+__device__ __forceinline__ rt_u32x4 rt_ld16(const uint8_t *p) { return *(const rt_u32x4_a8 *)p; }
+__device__ __forceinline__ rt_u32x2 rt_ld8(const uint8_t *p) { return *(const rt_u32x2_a4 *)p; }
+
+template <bool OPERAND>
+__global__ __launch_bounds__(256) void k_read_tiles(uint32_t *__restrict__ sink, const uint8_t *__restrict__ w,
+                                                    uint32_t n_sb) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t gx = gridDim.x;
+    // (workgroup ids go round the 8 XCDs: an XCD's tiles are contiguous, as in the decode kernels)
+    const uint32_t bx = (gx & 7u) == 0u ? (blockIdx.x & 7u) * (gx >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    const uint64_t row_bytes = (uint64_t)n_sb * 136u;
+    const uint8_t *tile = w + (uint64_t)bx * 16u * row_bytes;
+    const uint8_t *p0, *p1, *ps;
+    bool with_scales = true;
+    if (OPERAND) {
+        const uint8_t *row = tile + (lane & 15u) * row_bytes;
+        p0 = row + (lane >> 4) * 16u;
+        p1 = p0 + 64u;
+        ps = row + 128u;
+    } else {
+        p0 = tile + (lane >> 3) * row_bytes + (lane & 7u) * 16u;
+        p1 = p0 + 8u * row_bytes;
+        ps = tile + (lane & 15u) * row_bytes + 128u;
+        with_scales = lane < 16u;
+    }
+    rt_u32x4 a0[2], a1[2];
+    rt_u32x2 s[2] = {};
+    uint32_t acc = 0;
+    uint32_t sb = wave;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t b = min(sb + 4u * (uint32_t)i, n_sb - 1u) * 136u;
+        a0[i] = rt_ld16(p0 + b);
+        a1[i] = rt_ld16(p1 + b);
+        if (with_scales) s[i] = rt_ld8(ps + b);
+    }
+    for (; sb < n_sb; sb += 8u) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (sb + 4u * (uint32_t)i < n_sb)   // (uniform over the wave)
+                acc ^= a0[i].x ^ a0[i].y ^ a0[i].z ^ a0[i].w ^ a1[i].x ^ a1[i].y ^ a1[i].z ^ a1[i].w ^ s[i].x ^ s[i].y;
+            // (past the end of the row: its last super-block again, never folded in)
+            const uint32_t b = min(sb + 8u + 4u * (uint32_t)i, n_sb - 1u) * 136u;
+            a0[i] = rt_ld16(p0 + b);
+            a1[i] = rt_ld16(p1 + b);
+            if (with_scales) s[i] = rt_ld8(ps + b);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // (the last refills are never folded in: every byte of the tile counts once, the scales in
+    // operand order once per lane group)
+    for (int o = 32; o > 0; o >>= 1) acc ^= __shfl_xor(acc, o, 64);
+    if (lane == 0) sink[blockIdx.x * 4u + wave] = acc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -279,6 +346,22 @@ int dsx_synth_read_dev(void *stream, void *sink, const void *src, uint64_t bytes
     const uint32_t grid = (uint32_t)std::min<uint64_t>((n16 + 255) / 256, want);
     hipLaunchKernelGGL(k_read16, dim3(grid), dim3(256), 0, (hipStream_t)stream, (uint32_t *)sink,
                        (const uint4 *)src, n16);
+    return (int)hipGetLastError();
+}
+
+// Reads n_tiles 16-row tiles of an MXFP4 matrix with n_sb super-blocks per row (n_tiles * 16 * n_sb * 136
+// bytes at src) the way the decode kernels stream weights (see k_read_tiles); operand_order = 0: the
+// same bytes in memory order.  sink: 4 words per tile.
+int dsx_synth_read_tiles_dev(void *stream, void *sink, const void *src, uint32_t n_tiles, uint32_t n_sb,
+                             int operand_order) {
+    if (n_tiles == 0) return 0;
+    if (n_sb == 0 || (uintptr_t)src % 8u || (uintptr_t)sink % 4u) return (int)hipErrorInvalidValue;
+    if (operand_order)
+        hipLaunchKernelGGL(k_read_tiles<true>, dim3(n_tiles), dim3(256), 0, (hipStream_t)stream, (uint32_t *)sink,
+                           (const uint8_t *)src, n_sb);
+    else
+        hipLaunchKernelGGL(k_read_tiles<false>, dim3(n_tiles), dim3(256), 0, (hipStream_t)stream, (uint32_t *)sink,
+                           (const uint8_t *)src, n_sb);
     return (int)hipGetLastError();
 }
 

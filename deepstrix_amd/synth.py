@@ -42,6 +42,7 @@ def lib() -> C.CDLL:
         l.dsx_synth_q8_0_dev.argtypes = [vp, vp, u64, u64, u64, u64, u32, f32]
         l.dsx_synth_copy_dev.argtypes = [vp, vp, vp, u64]
         l.dsx_synth_read_dev.argtypes = [vp, vp, vp, u64, u32]
+        l.dsx_synth_read_tiles_dev.argtypes = [vp, vp, vp, u32, u32, C.c_int]
         _lib = l
     return _lib
 
@@ -115,3 +116,16 @@ def read_dev(sink, src, workgroups: int = 0) -> None:
                                   src.numel() * src.element_size(), workgroups)
     if rc:
         raise RuntimeError(f"dsx_synth_read_dev: hip error {rc}")
+
+
+def read_tiles_dev(sink, src, n_tiles: int, n_sb: int, operand_order: bool = True) -> None:
+    """Streams the first n_tiles 16-row tiles of an MXFP4 matrix (rows of n_sb super-blocks) the way
+    the decode kernels stream weights -- or, operand_order=False, the same bytes in memory order
+    (one word per wave into `sink`): the read rate that access pattern reaches on a device."""
+    import torch
+    assert src.numel() * src.element_size() >= n_tiles * 16 * n_sb * 136
+    assert sink.numel() * sink.element_size() >= 16 * n_tiles
+    rc = lib().dsx_synth_read_tiles_dev(torch.cuda.current_stream().cuda_stream, sink.data_ptr(), src.data_ptr(),
+                                        n_tiles, n_sb, 1 if operand_order else 0)
+    if rc:
+        raise RuntimeError(f"dsx_synth_read_tiles_dev: hip error {rc}")
