@@ -357,20 +357,14 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
         const uint32_t nj = (cnt + 15u) / 16u;  // column groups that hold a real column
         issue_phase(0, 0, 0);
         issue_yd(0);
-        // (On planar weights the LDS-direct loads fetch whole lines and the register ring loses: 1.36
-        // against 1.45 ms per layer at 512 tokens of the DeepSeek-V3 shape; on the engine's rows it wins,
-        // 1.73 against 1.80 ms, 1.34 against 1.40 at 128 tokens.)
-        constexpr bool kStream = !PLANAR;
-        if (nj > 4u || !kStream) {
 #pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
+        for (int r = 0; r < kGemmRF; r++)
 #pragma unroll
-                for (int m = 0; m < 2; m++)
+            for (int m = 0; m < 2; m++)
 #pragma unroll
-                    for (int j = 0; j < kGemmCG; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-        }
+                for (int j = 0; j < kGemmCG; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
 
         // One phase: NJP column groups, the first of them column group J0 of the tile.  ALoads
         // of the next super-block's weight loads, starting with load AFrom, go out one behind each
@@ -523,206 +517,16 @@ __global__ __launch_bounds__(kGemmWaves * 64, MT == kGemmMT ? 2 : 4) void k_mxfp
             for (; sb + 1u < p.n_sb; sb++) step_two_phases(njc, I1{}, sb);
             step_two_phases(njc, I0{}, sb);
         };
-        // ---- up to 64 columns on the engine's rows: the weights never see LDS --------------------
-        // A tile of a few columns has little to multiply per super-block, and its step is then the
-        // round trip of the weight loads that the step before it issued (one super-block of
-        // the 512 rows fills the weight region, so LDS cannot hold a second one in flight).  Here
-        // every lane loads its own operands -- row lane % 16, block lane / 16: the instruction's
-        // layout, as the decode kernels do -- into a ring of three super-blocks of registers
-        // (the 64 accumulator registers of the other four column groups are free), so that two
-        // super-blocks of weights are on their way while one is multiplied; the columns come through
-        // three of the phase buffers two steps ahead.  All loads of the loop are written out (the
-        // compiler sees none of them), and a wait names how many younger loads may stay in flight.
-        constexpr int kRing = 3;
-        struct AReg { u32x4_t a0, a1; u32x2_t s; };
-        AReg ring[kRing][kGemmRF][2];
-        // lane offsets from a fragment's first row: its nibble block (row n16, block g4), its scales
-        const uint32_t w_off = PLANAR ? n16 * p.n_sb * 128u + g4 * 16u : n16 * row_stride + g4 * 16u;
-        const uint32_t s_off = PLANAR ? p.n_sb * 2048u + n16 * 8u : n16 * row_stride + 128u;
-        auto issue_ring = [&](auto slotc, uint32_t sb) __attribute__((always_inline)) {
-            constexpr int slot = decltype(slotc)::value;
-            const uint32_t sbo = __builtin_amdgcn_readfirstlane(sb * kStepW);
-            const uint32_t wo = w_off, so = s_off;   // (copies: an asm operand alone does not capture)
-#pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    const uint8_t *base = wbase[m] + (a_slab[r][m] + sbo);
-                    u32x4_t v0, v1;
-                    u32x2_t vs;
-                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v0) : "v"(wo), "s"(base) : "memory");
-                    asm volatile("global_load_dwordx4 %0, %1, %2 offset:64" : "=v"(v1) : "v"(wo), "s"(base) : "memory");
-                    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(vs) : "v"(so), "s"(base) : "memory");
-                    ring[slot][r][m].a0 = v0;
-                    ring[slot][r][m].a1 = v1;
-                    ring[slot][r][m].s = vs;
-                }
-        };
-        constexpr int kRingLoads = 3 * 2 * kGemmRF;   // per wave and super-block
-        // everything but the loads of the two younger super-blocks has landed: the slot's registers
-        // (named, so that no use moves in front of the wait) and the wave's share of the columns
-        auto wait_ring = [&](auto slotc) __attribute__((always_inline)) {
-            constexpr int slot = decltype(slotc)::value;
-            static_assert(kGemmRF == 2, "the wait names the four fragments of a slot");
-            auto &R = ring[slot];   // (a reference first: an asm operand alone does not capture)
-            asm volatile("s_waitcnt vmcnt(%12)"
-                         : "+v"(R[0][0].a0), "+v"(R[0][0].a1), "+v"(R[0][0].s),
-                           "+v"(R[0][1].a0), "+v"(R[0][1].a1), "+v"(R[0][1].s),
-                           "+v"(R[1][0].a0), "+v"(R[1][0].a1), "+v"(R[1][0].s),
-                           "+v"(R[1][1].a0), "+v"(R[1][1].a1), "+v"(R[1][1].s)
-                         : "n"((kRing - 1) * kRingLoads)
-                         : "memory");
-        };
-        auto drain_ring = [&](auto slotc) __attribute__((always_inline)) {   // nothing of the slot is in flight any more
-            constexpr int slot = decltype(slotc)::value;
-            auto &R = ring[slot];
-            asm volatile("s_waitcnt vmcnt(0)"
-                         : "+v"(R[0][0].a0), "+v"(R[0][0].a1), "+v"(R[0][0].s),
-                           "+v"(R[0][1].a0), "+v"(R[0][1].a1), "+v"(R[0][1].s),
-                           "+v"(R[1][0].a0), "+v"(R[1][0].a1), "+v"(R[1][0].s),
-                           "+v"(R[1][1].a0), "+v"(R[1][1].a1), "+v"(R[1][1].s)
-                         :: "memory");
-        };
-        // the three column buffers of this loop: the two phase buffers and the start of the weight region
-        auto stream_buf = [&](uint32_t i) -> uint32_t {
-            return i == 0u ? 0u : i == 1u ? (uint32_t)kGemmPhaseBytes : (uint32_t)kGemmAOff;
-        };
-        auto issue_cols = [&](uint32_t sb, uint32_t bufoff) __attribute__((always_inline)) {
-            if (!ph_live[0]) return;
-            const uint8_t *src = p.act + __builtin_amdgcn_readfirstlane(sb * kStaged6Bytes);
-            const uint32_t dst = __builtin_amdgcn_readfirstlane(bp_lds + bufoff);
-            lds_dma16(dst, src, bp_fetch[0]);
-            lds_dma16(dst + (uint32_t)kGemmPhaseLine, src + 128, bp_fetch[0]);
-            lds_dma16(dst + 2u * (uint32_t)kGemmPhaseLine, src + 256, bp_fetch[0] ^ tflip);
-        };
-        // One super-block: NJ column groups against the slot's four fragments (as compute_phase),
-        // then the slot is requested again for the super-block three ahead.
-        auto stream_step = [&](auto njc, auto slotc, const uint32_t sb, const uint32_t bufoff) __attribute__((always_inline)) {
-            constexpr int NJ = decltype(njc)::value, slot = decltype(slotc)::value;
-            constexpr int NP = 4 * NJ;
-            wait_ring(slotc);
-            __syncthreads();   // every wave's columns of this super-block are there; the buffer two ahead is free
-            {
-                const uint32_t nb = sb + 2u < p.n_sb ? sb + 2u : p.n_sb - 1u;   // (past the end: the last one again)
-                const uint32_t i2 = (sb + 2u) % 3u;
-                issue_cols(nb, stream_buf(i2));
-                if (sb + 2u < p.n_sb) issue_yd(sb + 2u);
-            }
-            const uint8_t *pb = tiles + bufoff;
-            const float *yds = s_yd + ((sb >> 2) & 1u) * (uint32_t)(kYdBytes / 4) + (sb & 3u);
-            uint32_t sc[kGemmRF][2];
-#pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    const u32x2_t sv = ring[slot][r][m].s;
-                    sc[r][m] = ((sv.x >> (g4 * 8u)) & 0xFFu) | (((sv.y >> (g4 * 8u)) & 0xFFu) << 8);
-                }
-            auto load_piece = [&](int jj, int pp) __attribute__((always_inline)) -> v8i {   // pp = 2 half + plane
-                const int h = pp >> 1, q = pp & 1;
-                const uint4 hd = *(const uint4 *)(pb + (uint32_t)(h * kGemmPhaseLine + jj * 2048) + head_rd[q]);
-                const uint2 tl = *(const uint2 *)(pb + (uint32_t)(jj * 2048) + tail_rd[h][q]);
-                return v8i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w, (int)tl.x, (int)tl.y, 0, 0};
-            };
-            v4f c[kGemmRF][2];
-            v8i bring[2];
-            bring[0] = load_piece(0, 0);
-            float yd_prev = 0.0f, yd = 0.0f;
-            gemm_static_for<0, NP>([&](auto gpc) __attribute__((always_inline)) {
-                constexpr int gp = decltype(gpc)::value;
-                constexpr int jj = gp >> 2, pp = gp & 3, h = pp >> 1, q = pp & 1;
-                if (pp == 0) yd = yds[((uint32_t)jj * 16u + n16) * 4u];
-                if (gp + 1 < NP) bring[(gp + 1) & 1] = load_piece((gp + 1) >> 2, (gp + 1) & 3);
-                const v8i bq = bring[gp & 1];
-#pragma unroll
-                for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                    for (int m = 0; m < 2; m++) {
-                        const u32x4_t aw = h == 0 ? ring[slot][r][m].a0 : ring[slot][r][m].a1;
-                        const v8i av = {(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w, 0, 0, 0, 0};
-                        if (pp == 0) {
-                            if (jj > 0) {
-                                v4f &a = acc[r][m][jj > 0 ? jj - 1 : 0];
-                                a.x = fmaf(yd_prev, c[r][m].x, a.x);
-                                a.y = fmaf(yd_prev, c[r][m].y, a.y);
-                                a.z = fmaf(yd_prev, c[r][m].z, a.z);
-                                a.w = fmaf(yd_prev, c[r][m].w, a.w);
-                                asm volatile("" : "+v"(a));
-                            }
-                            c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                                av, bq, v4f{0.f, 0.f, 0.f, 0.f}, 4, 2, 0, (int)sc[r][m], 0, kScaleB6High);
-                        } else {
-                            c[r][m] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                                av, bq, c[r][m], 4, 2, h, (int)sc[r][m], 0, q == 0 ? kScaleB6High : kScaleB6Low);
-                        }
-                    }
-                if (pp == 3) yd_prev = yd;
-                asm volatile("" ::: "memory");
-                if constexpr (pp == 0 && jj > 0) {
-#pragma unroll
-                    for (int f = 0; f < 2 * kGemmRF; f++) {
-                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            });
-#pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++) {
-                    v4f &a = acc[r][m][NJ - 1];
-                    a.x = fmaf(yd_prev, c[r][m].x, a.x);
-                    a.y = fmaf(yd_prev, c[r][m].y, a.y);
-                    a.z = fmaf(yd_prev, c[r][m].z, a.z);
-                    a.w = fmaf(yd_prev, c[r][m].w, a.w);
-                    asm volatile("" : "+v"(a));
-                }
-            // (past the end: the last super-block again -- it is in the caches, nobody reads the
-            // registers, and every step issues the same number of loads, which the waits count on)
-            issue_ring(slotc, sb + (uint32_t)kRing < p.n_sb ? sb + (uint32_t)kRing : p.n_sb - 1u);
-        };
-        auto loop_stream = [&](auto njc) {
-            constexpr int NJ = decltype(njc)::value;
-#pragma unroll
-            for (int r = 0; r < kGemmRF; r++)
-#pragma unroll
-                for (int m = 0; m < 2; m++)
-#pragma unroll
-                    for (int j = 0; j < NJ; j++) acc[r][m][j] = v4f{0.f, 0.f, 0.f, 0.f};
-            // the columns of super-blocks 0 (requested above) and 1, then the ring
-            issue_cols(p.n_sb > 1u ? 1u : 0u, stream_buf(1u));
-            issue_ring(std::integral_constant<int, 0>{}, 0u);
-            issue_ring(std::integral_constant<int, 1>{}, p.n_sb > 1u ? 1u : 0u);
-            issue_ring(std::integral_constant<int, 2>{}, p.n_sb > 2u ? 2u : p.n_sb - 1u);
-            uint32_t boff = 0u;   // buffer of the current super-block: 0, 1, 2, 0, ...
-            auto next_buf = [&]() { boff = boff == 0u ? (uint32_t)kGemmPhaseBytes : boff == (uint32_t)kGemmPhaseBytes ? (uint32_t)kGemmAOff : 0u; };
-            for (uint32_t sb = 0; sb < p.n_sb; sb += (uint32_t)kRing) {
-                stream_step(njc, std::integral_constant<int, 0>{}, sb, boff);
-                next_buf();
-                if (sb + 1u < p.n_sb) {
-                    stream_step(njc, std::integral_constant<int, 1>{}, sb + 1u, boff);
-                    next_buf();
-                }
-                if (sb + 2u < p.n_sb) {
-                    stream_step(njc, std::integral_constant<int, 2>{}, sb + 2u, boff);
-                    next_buf();
-                }
-            }
-            drain_ring(std::integral_constant<int, 0>{});
-            drain_ring(std::integral_constant<int, 1>{});
-            drain_ring(std::integral_constant<int, 2>{});
-            __syncthreads();
-        };
-        auto loop_narrow = [&](auto njc) {
-            if constexpr (kStream) loop_stream(njc);
-            else loop_one_phase(njc);
-        };
+        // (A tile of up to 64 columns on the engine's rows used to run a loop of its own that took the
+        // weights through a ring of three super-blocks of registers in operand order instead of LDS:
+        // 4 % faster than this loop while it fetched a row's nibbles and scales apart, 5-7 % slower
+        // since it fetches them as one run -- 1.44 against 1.53 ms per layer at 256 tokens of the
+        // DeepSeek-V3 shape, 3.15 against 3.26 at 4096.)
         switch (nj) {
-            case 1: loop_narrow(std::integral_constant<int, 1>{}); break;
-            case 2: loop_narrow(std::integral_constant<int, 2>{}); break;
-            case 3: loop_narrow(std::integral_constant<int, 3>{}); break;
-            case 4: loop_narrow(std::integral_constant<int, 4>{}); break;
+            case 1: loop_one_phase(std::integral_constant<int, 1>{}); break;
+            case 2: loop_one_phase(std::integral_constant<int, 2>{}); break;
+            case 3: loop_one_phase(std::integral_constant<int, 3>{}); break;
+            case 4: loop_one_phase(std::integral_constant<int, 4>{}); break;
             case 5: loop_two_phases(std::integral_constant<int, 5>{}); break;
             case 6: loop_two_phases(std::integral_constant<int, 6>{}); break;
             case 7: loop_two_phases(std::integral_constant<int, 7>{}); break;

@@ -335,8 +335,8 @@ int dsx_moe_layer_set_profile_events(dsx_moe_layer *layer, void *gate_up_begin, 
  * from the layer's shape: which path a token count takes depends on the picks an expert receives,
  * T * n_used / n_expert (in brackets: the DeepSeek-V3 shape, 256 experts, top-8).
  * by_expert_chunk (1..16): token columns per work item of the small-batch by-expert path.
- * gemm_min_tokens (default for an all-MXFP4 layer: 16500 / sqrt(hidden * inter) picks per expert, held
- * within 3 .. 12 [4.3 picks: 138 tokens]; MXFP4 gate/up with a Q8_0 down matrix 2 [64], 4 for
+ * gemm_min_tokens (default for an all-MXFP4 layer: 3.5 picks per expert [112 tokens], 7 where
+ * n_expert * inter / 256 < 512; MXFP4 gate/up with a Q8_0 down matrix 2 [64], 4 for
  * matrices under 4 M elements; all-Q8_0 layers 1.5; on planar weights right behind the decode path
  * [17]): from this many tokens
  * on, a layer with MXFP4 gate/up runs the grouped-GEMM path (128 token columns per work item,

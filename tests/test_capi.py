@@ -179,16 +179,16 @@ def test_default_thresholds_follow_the_picks_per_expert():
     dsx_moe_layer_set_tuning): every shape gets its token counts from the ratios, none inherits the
     DeepSeek-V3 shape's."""
     v3 = _thresholds(7168, 2048, 256, 8)
-    # by-expert overtakes the decode launch at 13 .. 14 tokens, the GEMM the by-expert kernels at 128 .. 144
+    # by-expert overtakes the decode launch at 13 .. 14 tokens, the GEMM the by-expert kernels at 96 .. 128
     assert (v3["narrow"], v3["share"]) == (1, 4)
-    assert 13 <= v3["decode_max"] <= 14 and 129 <= v3["gemm"] <= 144
+    assert 13 <= v3["decode_max"] <= 14 and 97 <= v3["gemm"] <= 128
     # 128 experts, top-8, inter 1024: by-expert overtakes the decode launch between 12 and 16 tokens,
-    # the GEMM the by-expert kernels between 96 and 128
+    # the GEMM the by-expert kernels between 48 and 64
     e128 = _thresholds(4096, 1024, 128, 8)
-    assert 12 <= e128["decode_max"] <= 15 and 97 <= e128["gemm"] <= 129
-    # 64 experts, top-6, small matrices: 4 .. 5 tokens and 96 .. 128 tokens
+    assert 12 <= e128["decode_max"] <= 15 and 49 <= e128["gemm"] <= 64
+    # 64 experts, top-6, small matrices: 4 .. 5 tokens and 64 .. 96 tokens
     e64 = _thresholds(2048, 1536, 64, 6)
-    assert 4 <= e64["decode_max"] <= 5 and 97 <= e64["gemm"] <= 128
+    assert 4 <= e64["decode_max"] <= 5 and 65 <= e64["gemm"] <= 96
     # config 1 (all Q8_0): the int8 GEMM is ahead from 16 tokens on and far ahead at 24
     q8 = _thresholds(2048, 1408, 64, 6, capi.FMT_Q8_0, capi.FMT_Q8_0)
     assert 12 <= q8["gemm_q8"] <= 24
