@@ -165,19 +165,16 @@ static int fit_nt(uint32_t chunk, uint32_t n_blocks, int cap) {
 }
 
 
-// Group tables for many picks (two launches), with an optional extra group `n_expert` that
-// holds every token (slot n_used).
+// Group tables in one launch (a workgroup per group places its members, one more makes the counts,
+// offsets and work items: 3.5 us of kernel time up to a thousand picks, 10 us at 32768), with an
+// optional extra group `n_expert` that holds every token (slot n_used).
 int group_build_big(hipStream_t st, int32_t *group_count, int32_t *group_offset, int32_t *members,
                     int32_t *work_items, int32_t *n_work_items, const int32_t *selected, uint32_t b,
                     uint32_t n_used, uint32_t n_expert, uint32_t chunk, bool extra) {
-    hipLaunchKernelGGL(k_group_count, dim3(1), dim3(kGbThreads), 0, st, group_count, group_offset,
-                       work_items, n_work_items, selected, b, n_used, n_expert, chunk,
-                       extra ? 1u : 0u);
-    int rc = launched("group_count");
-    if (rc) return rc;
-    hipLaunchKernelGGL(k_group_scatter, dim3(n_expert + (extra ? 1u : 0u)), dim3(256), 0, st, members,
-                       group_count, group_offset, selected, b, n_used, n_expert);
-    return launched("group_scatter");
+    hipLaunchKernelGGL(k_group_tables, dim3(n_expert + (extra ? 1u : 0u) + 1u), dim3(kGbThreads), 0, st,
+                       group_count, group_offset, members, work_items, n_work_items, selected, b, n_used,
+                       n_expert, chunk, extra ? 1u : 0u);
+    return launched("group_tables");
 }
 
 // Grouped GEMM launch; max_wi bounds the number of work items, MT is the chunk they were built
@@ -461,15 +458,8 @@ static int group_build_impl(hipStream_t st, int32_t *group_count, int32_t *group
     if (b >= 65536 || n_used == 0 || n_used >= 65536)
         return fail(DSX_ERR_INVALID_ARG, "moe_group_build: b=%u n_used=%u must be below 65536", b, n_used);
     if (chunk == 0 || chunk > 128) return fail(DSX_ERR_INVALID_ARG, "moe_group_build: chunk=%u not in 1..128", chunk);
-    // many picks: histogram launch + one workgroup per expert (about 20 us whatever the count; the
-    // one-workgroup builder below takes 7 us + 0.044 us per pick)
-    if ((uint64_t)b * n_used > 320u)
-        return group_build_big(st, group_count, group_offset, expert_members, work_items,
-                               n_work_items, selected, b, n_used, n_expert, chunk, extra);
-    hipLaunchKernelGGL(k_group_build, dim3(1), dim3(kGbThreads), 0, st, group_count,
-                       group_offset, expert_members, work_items, n_work_items, selected, b, n_used,
-                       n_expert, chunk, extra ? 1u : 0u);
-    return launched("moe_group_build");
+    return group_build_big(st, group_count, group_offset, expert_members, work_items, n_work_items,
+                           selected, b, n_used, n_expert, chunk, extra);
 }
 
 int dsx_moe_group_build(dsx_stream_t stream, int32_t *group_count, int32_t *group_offset,

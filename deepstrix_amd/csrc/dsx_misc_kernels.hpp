@@ -572,9 +572,8 @@ __global__ __launch_bounds__(256) void k_q8_0_quantize(int8_t *__restrict__ xq,
 
 // ---------------------------------------------------------------------------------------
 // Token -> expert inversion: histogram, exclusive prefix sum, stable scatter, work items.
-// One workgroup of 1024 threads (b * n_used and n_expert are small next to the expert
-// products).  Members of an expert are in ascending (token, slot) order and work items in
-// ascending (expert, start) order, so the result is the same on every run.
+// Members of an expert are in ascending (token, slot) order and work items in ascending
+// (expert, start) order, so the result is the same on every run.
 // Replaces crates/v4flash-kernels/kernels/moe_group_builder.hip:32-51 and
 // moe_work_items_builder.hip:26-44 (atomic order, dense [n_expert x max] table).
 // ---------------------------------------------------------------------------------------
@@ -583,8 +582,8 @@ constexpr int kGbThreads = 1024;
 // Exclusive prefix sums of count[0..n) into off[0..n] and of the groups' work items,
 // ceil(count / chunk), into wi_off[0..n] (entry n: the totals), by the first wave of the workgroup:
 // a lane adds up its share of consecutive groups, the lanes scan their sums with shuffles, and
-// every lane writes its groups' offsets (one thread walking 257 groups through LDS took 8 us of the
-// builders' 17).  The caller puts a barrier on either side.
+// every lane writes its groups' offsets (one thread walking 257 groups through LDS took 8 us).
+// The caller puts a barrier on either side.
 __device__ __forceinline__ void gb_scan(const int *s_count, int *s_off, int *s_wi_off, uint32_t n,
                                         uint32_t chunk, uint32_t tid) {
     if (tid >= 64u) return;
@@ -618,77 +617,13 @@ __device__ __forceinline__ void gb_scan(const int *s_count, int *s_off, int *s_w
 }
 
 
-__global__ __launch_bounds__(kGbThreads) void k_group_build(
-    int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
-    int32_t *__restrict__ members, int32_t *__restrict__ work_items,
-    int32_t *__restrict__ n_work_items, const int32_t *__restrict__ selected, uint32_t b,
-    uint32_t n_used, uint32_t n_expert, uint32_t chunk, uint32_t extra) {
-    __shared__ int s_count[DSX_MAX_EXPERTS_K];
-    __shared__ int s_off[DSX_MAX_EXPERTS_K + 1];
-    __shared__ int s_wi_off[DSX_MAX_EXPERTS_K + 1];
-    // the picks, kept in LDS for the scatter below, which walks them once per expert (from global
-    // memory every walk step waits for a load: 44 ns per pick)
-    constexpr uint32_t kGbPicksInLds = 2048;
-    __shared__ int s_sel[kGbPicksInLds];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t total = b * n_used;
-    for (uint32_t e = tid; e < n_expert; e += kGbThreads) s_count[e] = 0;
-    __syncthreads();
-    for (uint32_t i = tid; i < total; i += kGbThreads) {
-        const int e = selected[i];
-        if (i < kGbPicksInLds) s_sel[i] = e;
-        if (e >= 0 && (uint32_t)e < n_expert) atomicAdd(&s_count[e], 1);
-    }
-    __syncthreads();
-    gb_scan(s_count, s_off, s_wi_off, n_expert, chunk, tid);
-    __syncthreads();
-    // the optional extra group n_expert: every token, slot n_used
-    if (tid == 0) *n_work_items = s_wi_off[n_expert] + (extra ? (int)((b + chunk - 1) / chunk) : 0);
-    if (extra) {
-        const uint32_t base = (uint32_t)s_off[n_expert], wbase = (uint32_t)s_wi_off[n_expert];
-        for (uint32_t t = tid; t < b; t += kGbThreads) members[base + t] = (int)((t << 16) | n_used);
-        for (uint32_t c = tid; c < (b + chunk - 1) / chunk; c += kGbThreads)
-            work_items[wbase + c] = (int)((n_expert << 16) | (c * chunk));
-        if (tid == 0) {
-            group_count[n_expert] = (int)b;
-            group_offset[n_expert + 1] = (int)(base + b);
-        }
-    }
-    for (uint32_t e = tid; e < n_expert; e += kGbThreads) {
-        group_count[e] = s_count[e];
-        group_offset[e] = s_off[e];
-        const int nwi = s_wi_off[e + 1] - s_wi_off[e];
-        for (int c = 0; c < nwi; c++)
-            work_items[s_wi_off[e] + c] = (int)((e << 16) | ((uint32_t)c * chunk));
-    }
-    if (tid == 0) group_offset[n_expert] = s_off[n_expert];
-    // stable scatter: a wave owns experts wave, wave + 16, ...; it walks the picks 64 at
-    // a time and places the matching ones with a ballot prefix count.
-    const uint32_t wave = tid >> 6, lane = tid & 63u;
-    for (uint32_t e = wave; e < n_expert; e += kGbThreads / 64) {
-        if (s_count[e] == 0) continue;
-        uint32_t pos = (uint32_t)s_off[e];
-        for (uint32_t i0 = 0; i0 < total; i0 += 64u) {
-            const uint32_t i = i0 + lane;
-            const bool hit = (i < total) && ((i < kGbPicksInLds ? s_sel[i] : selected[i]) == (int)e);
-            const uint64_t mask = __ballot(hit);
-            if (hit) {
-                const uint32_t before = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-                const uint32_t t = i / n_used, slot = i - t * n_used;
-                members[pos + before] = (int)((t << 16) | slot);
-            }
-            pos += (uint32_t)__popcll(mask);
-        }
-    }
-}
-
 // ---------------------------------------------------------------------------------------
-// The same tables for many picks, in two launches, plus an optional extra group with index
-// n_expert that every token belongs to (slot n_used): the dense expert riding along.
-//   k_group_count    one workgroup: histogram, prefix sums, work items
-//   k_group_scatter  one workgroup per expert: stable placement of that expert's members
+// The tables in one launch of n_groups + 1 workgroups, with an optional extra group of index
+// n_expert that every token belongs to (slot n_used): the dense expert riding along.  Workgroup n_groups makes the histogram, the prefix sums and the work items; workgroup
+// e < n_groups places the members of group e.  A placing workgroup reads every pick anyway, so it
+// counts the picks of lower groups itself (its group's offset) and waits for nobody.
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kGbThreads) void k_group_count(
+__device__ __forceinline__ void group_count_body(
     int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
     int32_t *__restrict__ work_items, int32_t *__restrict__ n_work_items,
     const int32_t *__restrict__ selected, uint32_t b, uint32_t n_used, uint32_t n_expert,
@@ -736,27 +671,28 @@ __global__ __launch_bounds__(kGbThreads) void k_group_count(
     }
 }
 
-__global__ __launch_bounds__(256) void k_group_scatter(int32_t *__restrict__ members,
-                                                       const int32_t *__restrict__ group_count,
-                                                       const int32_t *__restrict__ group_offset,
-                                                       const int32_t *__restrict__ selected,
-                                                       uint32_t b, uint32_t n_used,
-                                                       uint32_t n_expert) {
-    __shared__ uint32_t s_cnt[4];
-    const uint32_t e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t count = (uint32_t)group_count[e];
-    if (count == 0u) return;
-    const uint32_t base = (uint32_t)group_offset[e];
-    if (e >= n_expert) {  // the extra group: every token, slot n_used
-        for (uint32_t t = tid; t < b; t += 256u) members[base + t] = (int)((t << 16) | n_used);
+__global__ __launch_bounds__(kGbThreads) void k_group_tables(
+    int32_t *__restrict__ group_count, int32_t *__restrict__ group_offset,
+    int32_t *__restrict__ members, int32_t *__restrict__ work_items,
+    int32_t *__restrict__ n_work_items, const int32_t *__restrict__ selected, uint32_t b,
+    uint32_t n_used, uint32_t n_expert, uint32_t chunk, uint32_t extra) {
+    constexpr uint32_t kWaves = kGbThreads / 64;
+    __shared__ uint32_t s_mine[kWaves], s_below[kWaves];
+    const uint32_t n_groups = n_expert + (extra ? 1u : 0u);
+    if (blockIdx.x >= n_groups) {
+        group_count_body(group_count, group_offset, work_items, n_work_items, selected, b, n_used,
+                         n_expert, chunk, extra);
         return;
     }
-    // each wave owns a quarter of the picks (rounded to 256): count, then place; a lane looks at
+    const uint32_t e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    // picks that go in front of this group's members: the valid ones of lower groups (for the extra
+    // group e == n_expert: every valid pick)
+    // each wave owns a sixteenth of the picks (rounded to 256): count, then place; a lane looks at
     // four consecutive picks per step (one 16-byte load when `selected` is aligned for it)
     const uint32_t total = b * n_used;
     const bool vec = ((uintptr_t)selected & 15u) == 0u;
-    const uint32_t quarter = ((total + 1023u) / 1024u) * 256u;
-    const uint32_t i_begin = min(total, wave * quarter), i_end = min(total, i_begin + quarter);
+    const uint32_t share = ((total + 256u * kWaves - 1u) / (256u * kWaves)) * 256u;
+    const uint32_t i_begin = min(total, wave * share), i_end = min(total, i_begin + share);
     auto load4 = [&](uint32_t i0) -> int4 {  // picks i0 + 4 lane + j, -1 past the end
         const uint32_t i = i0 + lane * 4u;
         int4 q = {-1, -1, -1, -1};
@@ -770,19 +706,32 @@ __global__ __launch_bounds__(256) void k_group_scatter(int32_t *__restrict__ mem
         }
         return q;
     };
+    auto n_lanes = [](bool c) { return (uint32_t)__popcll(__ballot(c)); };
     // the next step's picks are requested before this step's are counted
-    uint32_t mine = 0;
+    uint32_t mine = 0, below = 0;
     int4 cur = load4(i_begin);
     for (uint32_t i0 = i_begin; i0 < i_end; i0 += 256u) {
         const int4 nxt = load4(i0 + 256u);
-        mine += (uint32_t)__popcll(__ballot(cur.x == (int)e)) + (uint32_t)__popcll(__ballot(cur.y == (int)e)) +
-                (uint32_t)__popcll(__ballot(cur.z == (int)e)) + (uint32_t)__popcll(__ballot(cur.w == (int)e));
+        mine += n_lanes(cur.x == (int)e) + n_lanes(cur.y == (int)e) + n_lanes(cur.z == (int)e) +
+                n_lanes(cur.w == (int)e);
+        // (a negative pick is a large unsigned number: never below)
+        below += n_lanes((uint32_t)cur.x < e) + n_lanes((uint32_t)cur.y < e) +
+                 n_lanes((uint32_t)cur.z < e) + n_lanes((uint32_t)cur.w < e);
         cur = nxt;
     }
-    if (lane == 0) s_cnt[wave] = mine;
+    if (lane == 0) {
+        s_mine[wave] = mine;
+        s_below[wave] = below;
+    }
     __syncthreads();
-    uint32_t pos = base;
-    for (uint32_t w = 0; w < wave; w++) pos += s_cnt[w];
+    uint32_t pos = 0;
+    for (uint32_t w = 0; w < kWaves; w++) pos += s_below[w] + (w < wave ? s_mine[w] : 0u);
+    if (e >= n_expert) {  // the extra group: every token, slot n_used, behind every valid pick
+        uint32_t base = 0;
+        for (uint32_t w = 0; w < kWaves; w++) base += s_below[w];
+        for (uint32_t t = tid; t < b; t += kGbThreads) members[base + t] = (int)((t << 16) | n_used);
+        return;
+    }
     if (mine == 0u) return;
     const uint64_t lower = (1ull << lane) - 1ull;
     cur = load4(i_begin);
